@@ -1,0 +1,115 @@
+/*
+ * C ABI of the gfx950 (MI355X / CDNA4) block-sparse FlashAttention-2 forward.
+ *
+ * This is the boundary a binding for the reference's operator would bind: plain
+ * pointers and sizes, no torch types.  The reference exposes the same operation
+ * through five pybind entry points that share one 13-argument signature
+ * (omni-attn-mma/pybind/omni_attn.cc:10-68, exported at :70-77); each of them
+ * unpacks its torch::Tensor arguments into exactly the pointer/size list below
+ * before launching (e.g. omni-attn-mma/mma/attn_naive.cu:317-402).
+ *
+ * All pointers are device pointers valid on the device that is current when the
+ * call is made.  Calls are asynchronous: work is enqueued on `stream` and the
+ * function returns without waiting.  No device memory is allocated or freed by
+ * any entry point and no state is kept between calls.
+ */
+#ifndef OMNI_ATTN_GFX950_H
+#define OMNI_ATTN_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element type of Q, K, V and O (fp32 accumulation in both cases). */
+enum omni_attn_dtype {
+  OMNI_ATTN_DTYPE_F16 = 0,
+  OMNI_ATTN_DTYPE_BF16 = 1
+};
+
+/* Block types, values fixed by omni-attn-mma/omni_attn_torch.py:38-41 and
+ * omni-attn-mma/mma/attn_naive.cu:4-7. */
+enum omni_attn_block_type {
+  OMNI_ATTN_BLOCK_MASKED = 0,
+  OMNI_ATTN_BLOCK_CAUSAL = 1,
+  OMNI_ATTN_BLOCK_FULL = 2,
+  OMNI_ATTN_BLOCK_PARTIAL = 3
+};
+
+/* Return codes.  0 is success; everything else leaves O untouched. */
+enum omni_attn_status {
+  OMNI_ATTN_OK = 0,
+  OMNI_ATTN_ERR_NULL_POINTER = 1,      /* a required pointer is NULL */
+  OMNI_ATTN_ERR_BAD_SHAPE = 2,         /* non-positive size, or Tq != ceil(S_pad / QB) */
+  OMNI_ATTN_ERR_UNSUPPORTED_HEAD_DIM = 3,   /* D not in {32, 64, 128} */
+  OMNI_ATTN_ERR_UNSUPPORTED_BLOCK = 4, /* QB or KB not in {64, 128} */
+  OMNI_ATTN_ERR_UNSUPPORTED_DTYPE = 5,
+  OMNI_ATTN_ERR_LAUNCH = 6,            /* hipLaunch failed; see omni_attn_last_hip_error() */
+  OMNI_ATTN_ERR_TOO_LARGE = 7          /* a tensor exceeds 2^31-1 elements per (b,h) slab */
+};
+
+/*
+ * Block-sparse attention forward:  for every (b, h) and every query block qb,
+ *   O[b,h,q,:] = softmax_k( mask(Q[b,h,q,:] . K[b,h,k,:] / sqrt(D)) ) V[b,h,k,:]
+ * over the KV blocks listed in kv_indices[b,h,qb,0:kv_num_blocks[b,h,qb]] only.
+ *
+ * Replaces the body of the reference's five launchers
+ *   omni_attn_simple_kernel                         (omni-attn-mma/mma/attn_naive.cu:305-408)
+ *   omni_attn_cp_async                              (omni-attn-mma/mma/omni_attn_cp_async.cu)
+ *   omni_attn_preftech_kernel                       (omni-attn-mma/mma/omni_attn_preftech.cu)
+ *   omni_attn_mma_stages_split_q_shared_kv          (omni-attn-mma/mma/omni_attn_shared_kv.cu:693-1009)
+ *   omni_attn_mma_stages_split_q_shared_kv_swizzle  (omni-attn-mma/mma/omni_attn_swizzle.cu:721-1036)
+ * with the mask semantics of the scalar kernel (omni-attn-mma/mma/attn_naive.cu:21-302):
+ *
+ *   q, k, v, o       [B, H, S_pad, D] row-major, 16-bit elements of type `dtype`.
+ *   lse_or_null      [B, H, S_pad] fp32 natural-log logsumexp of the masked, scaled
+ *                    scores of each row, or NULL to skip it (the reference has no such
+ *                    output).  Rows with no allowed key get -inf.
+ *   kv_num_blocks    [B, H, Tq] int32.
+ *   kv_indices       [B, H, Tq, max_blocks] int32, KV block index per slot.
+ *   block_mask_types [B, H, Tq, max_blocks] int32, omni_attn_block_type per slot.
+ *   partial_idx_or_null   [B, H, Tq, max_blocks] int32 index into partial_masks for
+ *                    PARTIAL slots (-1 = none), or NULL when has_partial is false.
+ *   partial_masks_or_null [P, QB, KB] one byte per element, 1 = attend, 0 = masked
+ *                    (torch.bool storage), row-major q_local*KB + k_local, or NULL.
+ *   Tq               number of query blocks, must equal ceil(S_pad / QB).
+ *   seqlen_orig      rows >= seqlen_orig are written as zeros (lse -inf); keys
+ *                    >= seqlen_orig are never attended (attn_naive.cu:64-72, :113).
+ *
+ * Semantics per slot: MASKED is skipped; FULL keeps everything; CAUSAL keeps
+ * k_global <= q_global; PARTIAL keeps the stored bytes; a PARTIAL slot whose
+ * partial pointers are NULL or whose index is negative is skipped
+ * (attn_naive.cu:119-131).  A row with no allowed key yields O = 0.
+ * The softmax scale is always 1/sqrt(D) (attn_naive.cu:88).
+ * Out-of-range metadata cannot fault the device: kv_num_blocks is clamped to
+ * [0, max_blocks] and kv_indices to [0, ceil(S_pad / KB) - 1].
+ *
+ * `stream` is a hipStream_t passed as void* (NULL = the legacy default stream).
+ */
+int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v, void* o,
+                         float* lse_or_null,
+                         const int32_t* kv_num_blocks,
+                         const int32_t* kv_indices,
+                         const int32_t* block_mask_types,
+                         const int32_t* partial_idx_or_null,
+                         const uint8_t* partial_masks_or_null,
+                         int B, int H, int S_pad, int D,
+                         int Tq, int max_blocks, int QB, int KB,
+                         int seqlen_orig, int dtype, void* stream);
+
+/* Static description of a return code (never NULL). */
+const char* omni_attn_status_string(int status);
+
+/* hipError_t of the most recent failed launch on the calling thread (0 if none). */
+int omni_attn_last_hip_error(void);
+
+/* Version of this ABI; bumped when a signature changes. */
+int omni_attn_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* OMNI_ATTN_GFX950_H */

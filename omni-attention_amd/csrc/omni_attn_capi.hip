@@ -1,0 +1,100 @@
+// C ABI of the forward: argument validation, instance dispatch, error codes.
+// Mirrors what the reference's launchers check before they launch
+// (omni-attn-mma/mma/attn_naive.cu:312-356, omni-attn-mma/mma/omni_attn_shared_kv.cu:701-768)
+// minus everything that is a property of torch tensors (dtype objects, contiguity),
+// which the binding layer above this file checks.
+#include "../../include/omni_attn_gfx950.h"
+#include "omni_attn_fwd_kernel.hpp"
+
+#include <cmath>
+
+namespace omni_attn {
+template <bool BF16, int D>
+int launch_fwd_blocks(const FwdParams& p, int QB, int KB, hipStream_t stream);
+template <> int launch_fwd_blocks<false, 32>(const FwdParams&, int, int, hipStream_t);
+template <> int launch_fwd_blocks<false, 64>(const FwdParams&, int, int, hipStream_t);
+template <> int launch_fwd_blocks<false, 128>(const FwdParams&, int, int, hipStream_t);
+template <> int launch_fwd_blocks<true, 32>(const FwdParams&, int, int, hipStream_t);
+template <> int launch_fwd_blocks<true, 64>(const FwdParams&, int, int, hipStream_t);
+template <> int launch_fwd_blocks<true, 128>(const FwdParams&, int, int, hipStream_t);
+}  // namespace omni_attn
+
+namespace {
+thread_local int g_last_hip_error = 0;
+}
+
+extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v, void* o,
+                                    float* lse_or_null, const int32_t* kv_num_blocks,
+                                    const int32_t* kv_indices, const int32_t* block_mask_types,
+                                    const int32_t* partial_idx_or_null,
+                                    const uint8_t* partial_masks_or_null, int B, int H, int S_pad,
+                                    int D, int Tq, int max_blocks, int QB, int KB, int seqlen_orig,
+                                    int dtype, void* stream) {
+  using namespace omni_attn;
+  if (!q || !k || !v || !o || !kv_num_blocks || !kv_indices || !block_mask_types)
+    return OMNI_ATTN_ERR_NULL_POINTER;
+  if (dtype != OMNI_ATTN_DTYPE_F16 && dtype != OMNI_ATTN_DTYPE_BF16)
+    return OMNI_ATTN_ERR_UNSUPPORTED_DTYPE;
+  if (D != 32 && D != 64 && D != 128) return OMNI_ATTN_ERR_UNSUPPORTED_HEAD_DIM;
+  if ((QB != 64 && QB != 128) || (KB != 64 && KB != 128)) return OMNI_ATTN_ERR_UNSUPPORTED_BLOCK;
+  if (B <= 0 || H <= 0 || S_pad <= 0 || Tq <= 0 || max_blocks <= 0 || seqlen_orig < 0)
+    return OMNI_ATTN_ERR_BAD_SHAPE;
+  if (Tq != (S_pad + QB - 1) / QB) return OMNI_ATTN_ERR_BAD_SHAPE;
+  const long long total = (long long)B * H * Tq;
+  if ((long long)S_pad * D > 0x7fffffffLL || total > 0x7fffffffLL - 8 ||
+      total * max_blocks > (1LL << 40))
+    return OMNI_ATTN_ERR_TOO_LARGE;
+
+  FwdParams p;
+  p.q = static_cast<const uint16_t*>(q);
+  p.k = static_cast<const uint16_t*>(k);
+  p.v = static_cast<const uint16_t*>(v);
+  p.o = static_cast<uint16_t*>(o);
+  p.lse = lse_or_null;
+  p.kv_num_blocks = kv_num_blocks;
+  p.kv_indices = kv_indices;
+  p.types = block_mask_types;
+  const bool has_partial = partial_idx_or_null != nullptr && partial_masks_or_null != nullptr;
+  p.partial_idx = has_partial ? partial_idx_or_null : nullptr;
+  p.partial_masks = has_partial ? partial_masks_or_null : nullptr;
+  p.S = S_pad;
+  p.Tq = Tq;
+  p.Tk = (S_pad + KB - 1) / KB;
+  p.max_blocks = max_blocks;
+  p.seqlen = seqlen_orig < S_pad ? seqlen_orig : S_pad;
+  p.total_work = int(total);
+  p.work_per_xcd = int((total + 7) / 8);
+  p.sl2 = float(1.4426950408889634 / std::sqrt(double(D)));
+
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool bf = dtype == OMNI_ATTN_DTYPE_BF16;
+  int err;
+  switch (D) {
+    case 32: err = bf ? launch_fwd_blocks<true, 32>(p, QB, KB, s) : launch_fwd_blocks<false, 32>(p, QB, KB, s); break;
+    case 64: err = bf ? launch_fwd_blocks<true, 64>(p, QB, KB, s) : launch_fwd_blocks<false, 64>(p, QB, KB, s); break;
+    default: err = bf ? launch_fwd_blocks<true, 128>(p, QB, KB, s) : launch_fwd_blocks<false, 128>(p, QB, KB, s); break;
+  }
+  if (err != 0) {
+    g_last_hip_error = err;
+    return OMNI_ATTN_ERR_LAUNCH;
+  }
+  return OMNI_ATTN_OK;
+}
+
+extern "C" const char* omni_attn_status_string(int status) {
+  switch (status) {
+    case OMNI_ATTN_OK: return "ok";
+    case OMNI_ATTN_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case OMNI_ATTN_ERR_BAD_SHAPE: return "bad shape: sizes must be positive and Tq == ceil(S_pad / Q_BLOCK_SIZE)";
+    case OMNI_ATTN_ERR_UNSUPPORTED_HEAD_DIM: return "unsupported head_dim (supported: 32, 64, 128)";
+    case OMNI_ATTN_ERR_UNSUPPORTED_BLOCK: return "unsupported Q_BLOCK_SIZE / KV_BLOCK_SIZE (supported: 64, 128)";
+    case OMNI_ATTN_ERR_UNSUPPORTED_DTYPE: return "unsupported dtype (supported: fp16, bf16)";
+    case OMNI_ATTN_ERR_LAUNCH: return "HIP kernel launch failed";
+    case OMNI_ATTN_ERR_TOO_LARGE: return "tensor too large for 32-bit slab indexing";
+    default: return "unknown status";
+  }
+}
+
+extern "C" int omni_attn_last_hip_error(void) { return g_last_hip_error; }
+
+extern "C" int omni_attn_abi_version(void) { return 1; }

@@ -1,0 +1,169 @@
+// Python module `omni_attn`: the operator surface the reference exports from
+// omni-attn-mma/pybind/omni_attn.cc:70-77 (five functions, one 13-argument positional
+// signature, :10-68), rebuilt over the gfx950 C ABI.  All five names run the same
+// kernel; `omni_attn_preftech` is the name the reference's own wrapper tries to import
+// (omni-attn-mma/omni_attn_torch.py:978), and `omni_attn_forward` additionally returns
+// the row logsumexp.
+//
+// Host-only C++: the device code lives behind include/omni_attn_gfx950.h.
+#include <torch/extension.h>
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include <stdexcept>
+#include <string>
+
+#include "omni_attn_gfx950.h"
+
+namespace {
+
+void check_qkvo(const torch::Tensor& t, const char* name, const torch::Tensor& q) {
+  if (!t.is_cuda()) throw std::runtime_error(std::string(name) + " must be a GPU tensor");
+  if (t.dim() != 4) throw std::runtime_error(std::string(name) + " must have shape [B, H, S, D]");
+  if (t.scalar_type() != q.scalar_type())
+    throw std::runtime_error(std::string("Tensor dtype mismatch: ") + name +
+                             " must have the dtype of Q (torch.float16 or torch.bfloat16)");
+  if (t.sizes() != q.sizes())
+    throw std::runtime_error(std::string(name) + " must have the shape of Q");
+  if (t.device() != q.device())
+    throw std::runtime_error(std::string(name) + " must be on the device of Q");
+}
+
+void check_meta(const torch::Tensor& t, const char* name, const torch::Tensor& q) {
+  if (t.scalar_type() != torch::kInt32)
+    throw std::runtime_error(std::string("Tensor dtype mismatch: ") + name + " must be torch.int32");
+  if (t.device() != q.device())
+    throw std::runtime_error(std::string(name) + " must be on the device of Q");
+}
+
+void forward_impl(const torch::Tensor& Q, const torch::Tensor& K, const torch::Tensor& V,
+                  torch::Tensor& O, float* lse, const torch::Tensor& kv_num_blocks,
+                  const torch::Tensor& kv_indices, const torch::Tensor& block_mask_types,
+                  int Q_BLOCK_SIZE, int KV_BLOCK_SIZE, int seqlen_orig,
+                  const torch::Tensor& partial_block_mask_indices,
+                  const torch::Tensor& partial_block_masks, bool has_partial) {
+  if (Q.scalar_type() != torch::kHalf && Q.scalar_type() != torch::kBFloat16)
+    throw std::runtime_error("Tensor dtype mismatch: Q must be torch.float16 or torch.bfloat16");
+  check_qkvo(Q, "Q", Q);
+  check_qkvo(K, "K", Q);
+  check_qkvo(V, "V", Q);
+  check_qkvo(O, "O", Q);
+  if (!Q.is_contiguous() || !K.is_contiguous() || !V.is_contiguous() || !O.is_contiguous())
+    throw std::runtime_error(
+        "Q, K, V, O tensors must be contiguous. Call .contiguous() before calling this function.");
+  check_meta(kv_num_blocks, "kv_num_blocks", Q);
+  check_meta(kv_indices, "kv_indices", Q);
+  check_meta(block_mask_types, "block_mask_types", Q);
+  if (!kv_num_blocks.is_contiguous() || !kv_indices.is_contiguous() ||
+      !block_mask_types.is_contiguous())
+    throw std::runtime_error(
+        "Block mask tensors must be contiguous. Call .contiguous() before calling this function.");
+
+  const int64_t B = Q.size(0), H = Q.size(1), S = Q.size(2), D = Q.size(3);
+  if (kv_num_blocks.dim() != 3 || kv_indices.dim() != 4 || block_mask_types.dim() != 4)
+    throw std::runtime_error(
+        "kv_num_blocks must be [B, H, num_q_blocks]; kv_indices and block_mask_types "
+        "[B, H, num_q_blocks, max_blocks]");
+  const int64_t num_q_blocks = kv_num_blocks.size(2);
+  const int64_t max_blocks = kv_indices.size(3);
+  if (Q_BLOCK_SIZE <= 0 || KV_BLOCK_SIZE <= 0)
+    throw std::runtime_error("Q_BLOCK_SIZE and KV_BLOCK_SIZE must be positive");
+  const int64_t expected = (S + Q_BLOCK_SIZE - 1) / Q_BLOCK_SIZE;
+  if (num_q_blocks != expected)
+    throw std::runtime_error("Block mask num_q_blocks (" + std::to_string(num_q_blocks) +
+                             ") does not match expected value (" + std::to_string(expected) +
+                             ") based on seqlen=" + std::to_string(S) +
+                             " and Q_BLOCK_SIZE=" + std::to_string(Q_BLOCK_SIZE));
+  if (kv_num_blocks.size(0) != B || kv_num_blocks.size(1) != H || kv_indices.size(0) != B ||
+      kv_indices.size(1) != H || kv_indices.size(2) != num_q_blocks ||
+      block_mask_types.sizes() != kv_indices.sizes())
+    throw std::runtime_error("Block mask tensor shapes do not match Q's batch / heads / blocks");
+
+  const int32_t* pidx = nullptr;
+  const uint8_t* pmask = nullptr;
+  if (has_partial) {
+    if (partial_block_mask_indices.scalar_type() != torch::kInt32)
+      throw std::runtime_error(
+          "Tensor dtype mismatch: partial_block_mask_indices must be torch.int32");
+    if (partial_block_masks.scalar_type() != torch::kBool)
+      throw std::runtime_error("Tensor dtype mismatch: partial_block_masks must be torch.bool");
+    if (!partial_block_mask_indices.is_contiguous() || !partial_block_masks.is_contiguous())
+      throw std::runtime_error("Partial block mask tensors must be contiguous.");
+    if (partial_block_mask_indices.sizes() != kv_indices.sizes())
+      throw std::runtime_error("partial_block_mask_indices must have the shape of kv_indices");
+    if (partial_block_masks.dim() != 3 || partial_block_masks.size(1) != Q_BLOCK_SIZE ||
+        partial_block_masks.size(2) != KV_BLOCK_SIZE)
+      throw std::runtime_error(
+          "partial_block_masks must be [num_partial, Q_BLOCK_SIZE, KV_BLOCK_SIZE]");
+    if (partial_block_mask_indices.device() != Q.device() ||
+        partial_block_masks.device() != Q.device())
+      throw std::runtime_error("Partial block mask tensors must be on the device of Q");
+    if (partial_block_masks.size(0) > 0) {
+      pidx = partial_block_mask_indices.data_ptr<int32_t>();
+      pmask = reinterpret_cast<const uint8_t*>(partial_block_masks.data_ptr<bool>());
+    }
+  }
+
+  c10::DeviceGuard guard(Q.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStream(Q.device().index()).stream();
+  const int dtype = Q.scalar_type() == torch::kBFloat16 ? OMNI_ATTN_DTYPE_BF16 : OMNI_ATTN_DTYPE_F16;
+  const int rc = omni_attn_fwd_gfx950(
+      Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), lse,
+      kv_num_blocks.data_ptr<int32_t>(), kv_indices.data_ptr<int32_t>(),
+      block_mask_types.data_ptr<int32_t>(), pidx, pmask, int(B), int(H), int(S), int(D),
+      int(num_q_blocks), int(max_blocks), Q_BLOCK_SIZE, KV_BLOCK_SIZE, seqlen_orig, dtype,
+      static_cast<void*>(stream));
+  if (rc != OMNI_ATTN_OK) {
+    std::string msg = std::string("omni_attn: ") + omni_attn_status_string(rc);
+    if (rc == OMNI_ATTN_ERR_UNSUPPORTED_HEAD_DIM) msg += ", got head_dim=" + std::to_string(D);
+    if (rc == OMNI_ATTN_ERR_UNSUPPORTED_BLOCK)
+      msg += ", got Q_BLOCK_SIZE=" + std::to_string(Q_BLOCK_SIZE) +
+             " KV_BLOCK_SIZE=" + std::to_string(KV_BLOCK_SIZE);
+    if (rc == OMNI_ATTN_ERR_LAUNCH)
+      msg += " (hipError " + std::to_string(omni_attn_last_hip_error()) + ")";
+    throw std::runtime_error(msg);
+  }
+}
+
+// The reference's signature: tensors by value, void return.
+void omni_attn_op(torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch::Tensor O,
+                  torch::Tensor kv_num_blocks, torch::Tensor kv_indices,
+                  torch::Tensor block_mask_types, int Q_BLOCK_SIZE, int KV_BLOCK_SIZE,
+                  int seqlen_orig, torch::Tensor partial_block_mask_indices,
+                  torch::Tensor partial_block_masks, bool has_partial) {
+  forward_impl(Q, K, V, O, nullptr, kv_num_blocks, kv_indices, block_mask_types, Q_BLOCK_SIZE,
+               KV_BLOCK_SIZE, seqlen_orig, partial_block_mask_indices, partial_block_masks,
+               has_partial);
+}
+
+// Same arguments plus LSE [B, H, S] fp32, written in place.
+void omni_attn_forward(torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch::Tensor O,
+                       torch::Tensor LSE, torch::Tensor kv_num_blocks, torch::Tensor kv_indices,
+                       torch::Tensor block_mask_types, int Q_BLOCK_SIZE, int KV_BLOCK_SIZE,
+                       int seqlen_orig, torch::Tensor partial_block_mask_indices,
+                       torch::Tensor partial_block_masks, bool has_partial) {
+  if (LSE.scalar_type() != torch::kFloat32)
+    throw std::runtime_error("Tensor dtype mismatch: LSE must be torch.float32");
+  if (!LSE.is_contiguous() || LSE.dim() != 3 || Q.dim() != 4 || LSE.size(0) != Q.size(0) ||
+      LSE.size(1) != Q.size(1) || LSE.size(2) != Q.size(2) || LSE.device() != Q.device())
+    throw std::runtime_error("LSE must be a contiguous [B, H, S] tensor on the device of Q");
+  forward_impl(Q, K, V, O, LSE.data_ptr<float>(), kv_num_blocks, kv_indices, block_mask_types,
+               Q_BLOCK_SIZE, KV_BLOCK_SIZE, seqlen_orig, partial_block_mask_indices,
+               partial_block_masks, has_partial);
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.doc() = "gfx950 block-sparse FlashAttention-2 forward (omni-attention operator surface)";
+  m.def("omni_attn_mma_stages_split_q_shared_kv", &omni_attn_op,
+        "omni_attn_mma_stages_split_q_shared_kv");
+  m.def("omni_attn_simple_kernel", &omni_attn_op, "omni_attn_simple_kernel");
+  m.def("omni_attn_cp_async", &omni_attn_op, "omni_attn_cp_async");
+  m.def("omni_attn_preftech_kernel", &omni_attn_op, "omni_attn_preftech_kernel");
+  m.def("omni_attn_preftech", &omni_attn_op, "omni_attn_preftech");
+  m.def("omni_attn_mma_stages_split_q_shared_kv_swizzle", &omni_attn_op,
+        "omni_attn_mma_stages_split_q_shared_kv_swizzle");
+  m.def("omni_attn_forward", &omni_attn_forward, "omni_attn_forward (also writes logsumexp)");
+  m.def("abi_version", []() { return omni_attn_abi_version(); });
+}
