@@ -1,0 +1,93 @@
+"""ctypes binding of the C ABI in include/omni_attn_gfx950.h.
+
+This is the stub a Python caller that does not want the torch extension module would
+write: it hands raw device pointers and sizes to ``libomni_attn_gfx950.so``.  Tensors
+are only used here as owners of device memory.  There is no fallback: a missing
+library raises ``OSError`` on first use.
+"""
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libomni_attn_gfx950.so")
+
+DTYPE_F16 = 0
+DTYPE_BF16 = 1
+
+EXPORTED_SYMBOLS = (
+    "omni_attn_fwd_gfx950",
+    "omni_attn_status_string",
+    "omni_attn_last_hip_error",
+    "omni_attn_abi_version",
+)
+
+_lib = None
+
+
+def load_library() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        lib = ctypes.CDLL(LIB_PATH)
+        vp, i32 = ctypes.c_void_p, ctypes.c_int
+        lib.omni_attn_fwd_gfx950.restype = i32
+        lib.omni_attn_fwd_gfx950.argtypes = [vp] * 10 + [i32] * 10 + [vp]
+        lib.omni_attn_status_string.restype = ctypes.c_char_p
+        lib.omni_attn_status_string.argtypes = [i32]
+        lib.omni_attn_last_hip_error.restype = i32
+        lib.omni_attn_abi_version.restype = i32
+        _lib = lib
+    return _lib
+
+
+def status_string(code: int) -> str:
+    return load_library().omni_attn_status_string(int(code)).decode()
+
+
+def _ptr(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def fwd_raw(q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, nb_ptr, idx_ptr, types_ptr, pidx_ptr, pmask_ptr,
+            B, H, S_pad, D, Tq, max_blocks, QB, KB, seqlen_orig, dtype, stream_ptr) -> int:
+    """The C call itself; returns the status code."""
+    return load_library().omni_attn_fwd_gfx950(
+        q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, nb_ptr, idx_ptr, types_ptr, pidx_ptr, pmask_ptr,
+        B, H, S_pad, D, Tq, max_blocks, QB, KB, seqlen_orig, dtype, stream_ptr)
+
+
+def fwd(q, k, v, o, lse, kv_num_blocks, kv_indices, block_mask_types, QB, KB, seqlen_orig,
+        partial_idx=None, partial_masks=None, stream: Optional[int] = None) -> None:
+    """Enqueue the forward on ``stream`` (default: torch's current stream of q's device).
+    q, k, v, o: contiguous [B, H, S_pad, D] fp16 or bf16 on the GPU; lse: fp32 [B, H, S_pad]
+    or None.  Raises RuntimeError with the library's message on a non-zero status."""
+    B, H, S, D = q.shape
+    for t in (q, k, v, o):
+        if not (t.is_cuda and t.is_contiguous() and t.dtype == q.dtype and t.shape == q.shape):
+            raise RuntimeError("q, k, v, o must be contiguous GPU tensors of one shape and dtype")
+    if q.dtype == torch.bfloat16:
+        dtype = DTYPE_BF16
+    elif q.dtype == torch.float16:
+        dtype = DTYPE_F16
+    else:
+        raise RuntimeError("q must be torch.float16 or torch.bfloat16")
+    for t in (kv_num_blocks, kv_indices, block_mask_types) + ((partial_idx,) if partial_idx is not None else ()):
+        if not (t.is_cuda and t.is_contiguous() and t.dtype == torch.int32):
+            raise RuntimeError("block-mask tensors must be contiguous int32 GPU tensors")
+    if partial_masks is not None:
+        if not (partial_masks.is_cuda and partial_masks.is_contiguous()
+                and partial_masks.dtype in (torch.bool, torch.uint8)):
+            raise RuntimeError("partial_masks must be a contiguous bool GPU tensor")
+        if partial_masks.numel() == 0:
+            partial_idx, partial_masks = None, None
+    if stream is None:
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+    with torch.cuda.device(q.device):
+        rc = fwd_raw(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(kv_num_blocks),
+                     _ptr(kv_indices), _ptr(block_mask_types), _ptr(partial_idx), _ptr(partial_masks),
+                     B, H, S, D, kv_num_blocks.shape[2], kv_indices.shape[3], QB, KB,
+                     int(seqlen_orig), dtype, stream)
+    if rc != 0:
+        raise RuntimeError("omni_attn_fwd_gfx950: %s (status %d)" % (status_string(rc), rc))

@@ -1,0 +1,93 @@
+"""fp32 dense-mask attention oracle (test infrastructure, see oracle/__init__.py).
+
+Follows naive_attention_with_dense_mask (omni-attn-mma/omni_attn_torch.py:348-387):
+scores = Q K^T / sqrt(D), masked positions -> -inf, softmax in fp32, times V.  Run in
+fp32 the reference's cast of the weights to the query dtype (:384) is the identity.
+Adds the row logsumexp and the kernels' convention for rows with no allowed key:
+output 0 (omni-attn-mma/mma/attn_naive.cu:177-183), logsumexp -inf.
+"""
+import math
+from typing import Optional, Tuple
+
+import torch
+
+
+def attention_dense_fp32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                         mask: torch.Tensor, row_chunk: int = 2048) -> Tuple[torch.Tensor, torch.Tensor]:
+    """q, k, v: [..., S, D] (any float dtype, converted to fp32 as they are);
+    mask: bool, broadcastable to [..., S, S], True = attend.
+    Returns (O fp32 [..., S, D], LSE fp32 [..., S])."""
+    qf, kf, vf = q.float(), k.float(), v.float()
+    S, D = qf.shape[-2], qf.shape[-1]
+    scale = 1.0 / math.sqrt(D)
+    out = torch.empty(qf.shape[:-1] + (vf.shape[-1],), dtype=torch.float32, device=qf.device)
+    lse = torch.empty(qf.shape[:-1], dtype=torch.float32, device=qf.device)
+    for r0 in range(0, S, row_chunk):
+        r1 = min(S, r0 + row_chunk)
+        s = torch.matmul(qf[..., r0:r1, :], kf.transpose(-1, -2)) * scale
+        m = mask[..., r0:r1, :]
+        s = s.masked_fill(~m, float("-inf"))
+        any_row = m.any(-1)
+        l = torch.logsumexp(s, dim=-1)
+        # softmax of an all -inf row is NaN in torch; those rows are defined as 0
+        p = torch.softmax(s, dim=-1)
+        p = torch.where(any_row.unsqueeze(-1), p, torch.zeros_like(p))
+        out[..., r0:r1, :] = torch.matmul(p, vf)
+        lse[..., r0:r1] = torch.where(any_row, l, torch.full_like(l, float("-inf")))
+    return out, lse
+
+
+def prefix_mask(prefix_len: torch.Tensor, kv_len: int) -> torch.Tensor:
+    """allow[..., i, j] = j < prefix_len[..., i]."""
+    j = torch.arange(kv_len, device=prefix_len.device)
+    return j < prefix_len.unsqueeze(-1)
+
+
+def transfusion_mask_bruteforce(seq_len: int, spans) -> torch.Tensor:
+    """Token rule of transfusion_pytorch/transfusion.py:496-515 written as loops:
+    allow[i, j] = (i >= j) or any span (off, length): i >= off and j < off + length."""
+    allow = torch.zeros(seq_len, seq_len, dtype=torch.bool)
+    for i in range(seq_len):
+        for j in range(seq_len):
+            ok = i >= j
+            for off, length in spans:
+                if i >= off and j < off + length:
+                    ok = True
+            allow[i, j] = ok
+    return allow
+
+
+def dense_mask_from_blocks(kv_num_blocks, kv_indices, block_mask_types, QB: int, KB: int,
+                           q_len: int, kv_len: int, partial_idx=None, partial_masks=None,
+                           seqlen_orig: Optional[int] = None) -> torch.Tensor:
+    """Dense mask the kernels realise for given block metadata, as plain loops over the
+    slots (scalar-kernel semantics, omni-attn-mma/mma/attn_naive.cu:95-175): MASKED and
+    PARTIAL-without-bits slots are skipped, CAUSAL is k_global <= q_global, keys and
+    rows at or beyond seqlen_orig are dropped."""
+    B, H, Tq, _ = kv_indices.shape
+    seqlen = q_len if seqlen_orig is None else min(seqlen_orig, q_len)
+    dense = torch.zeros(B, H, q_len, kv_len, dtype=torch.bool)
+    nb = kv_num_blocks.tolist()
+    idx = kv_indices.tolist()
+    tys = block_mask_types.tolist()
+    pid = partial_idx.tolist() if partial_idx is not None else None
+    for b in range(B):
+        for h in range(H):
+            for qb in range(Tq):
+                q0, q1 = qb * QB, min(qb * QB + QB, q_len)
+                for s in range(nb[b][h][qb]):
+                    kb, ty = idx[b][h][qb][s], tys[b][h][qb][s]
+                    k0, k1 = kb * KB, min(kb * KB + KB, kv_len)
+                    if ty == 2:
+                        dense[b, h, q0:q1, k0:k1] = True
+                    elif ty == 1:
+                        qq = torch.arange(q0, q1).view(-1, 1)
+                        kk = torch.arange(k0, k1).view(1, -1)
+                        dense[b, h, q0:q1, k0:k1] = kk <= qq
+                    elif ty == 3:
+                        if pid is None or partial_masks is None or pid[b][h][qb][s] < 0:
+                            continue
+                        dense[b, h, q0:q1, k0:k1] = partial_masks[pid[b][h][qb][s]][: q1 - q0, : k1 - k0]
+    dense[:, :, seqlen:, :] = False
+    dense[:, :, :, seqlen:] = False
+    return dense

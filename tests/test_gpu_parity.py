@@ -1,0 +1,181 @@
+"""Parity of the gfx950 kernel with the CPU oracle, called through the C ABI.
+
+Bars (written here, enforced in helpers.compare_with_oracle): max-abs on the output
+2e-3 for fp16 and 1e-2 for bf16, 1e-3 on the logsumexp, rows with no allowed key
+exactly 0 / -inf.  Inputs are rounded to the 16-bit type once; kernel and oracle see
+the same rounded values.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import omni_attn_capi
+from baseline_configs import make_workload
+from helpers import (HERE, TOL_LSE, TOL_O, compare_with_oracle, random_block_metadata)
+from oracle.block_walk import attention_block_walk
+from oracle.dense_oracle import attention_dense_fp32, dense_mask_from_blocks, prefix_mask
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(t, device):
+    return None if t is None else t.to(device).contiguous()
+
+
+def run_kernel(q, k, v, nb, idx, tys, QB, KB, seqlen, pidx=None, pm=None, device="cuda:0",
+               want_lse=True, stream=None):
+    """One forward through the C ABI.  O and LSE start as NaN so that any element the
+    kernel does not write shows up."""
+    qd, kd, vd = (_dev(t, device) for t in (q, k, v))
+    o = torch.full_like(qd, float("nan"))
+    lse = torch.full(qd.shape[:3], float("nan"), dtype=torch.float32, device=device) if want_lse else None
+    omni_attn_capi.fwd(qd, kd, vd, o, lse, _dev(nb, device), _dev(idx, device), _dev(tys, device), QB, KB,
+                       seqlen, _dev(pidx, device), _dev(pm, device), stream=stream)
+    torch.cuda.synchronize()
+    return o, lse
+
+
+def run_workload(w, device, **kw):
+    m = w.block_mask
+    return run_kernel(w.q, w.k, w.v, m.kv_num_blocks, m.kv_indices, m.block_mask_types, m.Q_BLOCK_SIZE,
+                      m.KV_BLOCK_SIZE, w.q.shape[2], m.partial_block_mask_indices, m.partial_block_masks,
+                      device=device, **kw)
+
+
+def test_c1_causal_full_parity(gpu_device):
+    w = make_workload("c1_causal", seed=0)
+    o, lse = run_workload(w, gpu_device)
+    S = 512
+    ro, rl = attention_dense_fp32(w.q, w.k, w.v, prefix_mask(w.prefix_len, S).unsqueeze(1))
+    compare_with_oracle(o, lse, ro, rl, torch.float16, "c1 vs dense oracle")
+    m = w.block_mask
+    wo, wl = attention_block_walk(w.q, w.k, w.v, m.kv_num_blocks, m.kv_indices, m.block_mask_types, 128, 128, S)
+    compare_with_oracle(o, lse, wo, wl, torch.float16, "c1 vs block walk")
+    gold = np.load(os.path.join(HERE, "golden", "c1_causal_seed0.npz"))
+    assert abs(float(gold["q_checksum"]) - w.q.double().sum().item()) < 1e-9, "inputs differ from the fixture's"
+    compare_with_oracle(o, lse, torch.from_numpy(gold["o"]), torch.from_numpy(gold["lse"]), torch.float16,
+                        "c1 vs committed fixture")
+    # causal row 0 attends key 0 only: O = V[0] bit for bit, lse = q0.k0/sqrt(D)
+    assert torch.equal(o[0, :, 0].cpu(), w.v[0, :, 0])
+
+
+def _merge_property(w, o, lse, device):
+    """Size-independent check over every head at full size: attention over a block list
+    equals the logsumexp-weighted merge of attention over its two halves."""
+    m = w.block_mask
+    nb = m.kv_num_blocks
+    half = nb // 2
+    max_blocks = m.kv_indices.shape[-1]
+    slot = torch.arange(max_blocks).view(1, 1, 1, -1)
+    # second half: shift the slots left by `half`
+    src = (slot + half.unsqueeze(-1).long()).clamp(max=max_blocks - 1)
+    def shifted(t):
+        return None if t is None else torch.gather(t, -1, src).contiguous()
+    QB, KB, S = m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, w.q.shape[2]
+    oa, la = run_kernel(w.q, w.k, w.v, half.contiguous(), m.kv_indices, m.block_mask_types, QB, KB, S,
+                        m.partial_block_mask_indices, m.partial_block_masks, device=device)
+    ob, lb = run_kernel(w.q, w.k, w.v, (nb - half).contiguous(), shifted(m.kv_indices),
+                        shifted(m.block_mask_types), QB, KB, S, shifted(m.partial_block_mask_indices),
+                        m.partial_block_masks, device=device)
+    l_merged = torch.logaddexp(la, lb)
+    wa = torch.exp(la - l_merged).nan_to_num(0.0).unsqueeze(-1)
+    wb = torch.exp(lb - l_merged).nan_to_num(0.0).unsqueeze(-1)
+    o_merged = wa * oa.float() + wb * ob.float()
+    live = ~torch.isinf(lse)
+    assert torch.equal(torch.isinf(l_merged), torch.isinf(lse))
+    assert (l_merged[live] - lse[live]).abs().max().item() <= TOL_LSE
+    # three roundings to the 16-bit type are involved instead of one
+    assert (o_merged - o.float()).abs().max().item() <= 2 * TOL_O[w.dtype]
+
+
+@pytest.mark.parametrize("name", ["c2_interleaved", "c2_interleaved_8k", "c3_partial", "c4_long",
+                                  "c5_batched", "c5_full_control"])
+def test_config_full_size(name, gpu_device):
+    """Full-size run; oracle on sampled (batch, head) slabs; merge property on all heads."""
+    w = make_workload(name, seed=0)
+    B, H, S, D = w.q.shape
+    o, lse = run_workload(w, gpu_device)
+    assert not torch.isnan(o).any() and not torch.isnan(lse).any()
+    samples = sorted({(0, 0), (B - 1, H - 1), (B // 2, H // 2)})
+    if name.startswith("c5"):
+        samples = sorted({(0, 0), (1, 1), (2, H - 1)}) if name == "c5_batched" else [(B - 1, 3)]
+    for b, h in samples:
+        mask = prefix_mask(w.prefix_len[b], S)
+        ro, rl = attention_dense_fp32(w.q[b, h], w.k[b, h], w.v[b, h], mask)
+        compare_with_oracle(o[b, h], lse[b, h], ro, rl, w.dtype, f"{name} slab ({b},{h})")
+    _merge_property(w, o, lse, gpu_device)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("QB,KB", [(128, 128), (128, 64), (64, 128), (64, 64)])
+def test_random_metadata_all_slot_kinds(dtype, D, QB, KB, gpu_device):
+    """FULL / CAUSAL (on and off the diagonal) / PARTIAL with bits / PARTIAL without bits /
+    MASKED slots, unordered kv_indices, empty query blocks, fully masked rows inside
+    listed blocks, for every (Q_BLOCK, KV_BLOCK, head_dim, dtype) instance."""
+    gen = torch.Generator().manual_seed(1000 * D + 10 * QB + KB)
+    B, H, S = 2, 2, 512
+    q, k, v = (torch.randn(B, H, S, D, generator=gen).to(dtype) for _ in range(3))
+    nb, idx, tys, pidx, pm = random_block_metadata(gen, B, H, S // QB, S // KB, QB, KB, shuffle=True)
+    for seqlen in (S, S - 45):
+        o, lse = run_kernel(q, k, v, nb, idx, tys, QB, KB, seqlen, pidx, pm, device=gpu_device)
+        dense = dense_mask_from_blocks(nb, idx, tys, QB, KB, S, S, pidx, pm, seqlen_orig=seqlen)
+        ro, rl = attention_dense_fp32(q, k, v, dense)
+        compare_with_oracle(o, lse, ro, rl, dtype, f"dense oracle seqlen={seqlen}")
+        wo, wl = attention_block_walk(q, k, v, nb, idx, tys, QB, KB, seqlen, pidx, pm)
+        compare_with_oracle(o, lse, wo, wl, dtype, f"block walk seqlen={seqlen}")
+        assert (o[:, :, seqlen:] == 0).all()
+
+
+def test_lse_pointer_is_optional(gpu_device):
+    w = make_workload("c1_causal", seed=1)
+    o1, _ = run_workload(w, gpu_device)
+    o2, none = run_workload(w, gpu_device, want_lse=False)
+    assert none is None and torch.equal(o1, o2)
+
+
+def test_sequence_not_a_multiple_of_the_block(gpu_device):
+    """S_pad = 500 handed to the C ABI as it is (Tq = ceil(500/128) = 4): loads are clamped,
+    keys and rows beyond 500 do not exist."""
+    gen = torch.Generator().manual_seed(11)
+    S, D, QB, KB = 500, 64, 128, 64
+    q, k, v = (torch.randn(1, 3, S, D, generator=gen).to(torch.bfloat16) for _ in range(3))
+    from omni_attn_torch import create_causal_omni_block_mask
+    m = create_causal_omni_block_mask(1, 3, S, S, QB, KB, device="cpu")
+    o, lse = run_kernel(q, k, v, m.kv_num_blocks, m.kv_indices, m.block_mask_types, QB, KB, S, device=gpu_device)
+    ro, rl = attention_dense_fp32(q, k, v, torch.tril(torch.ones(S, S, dtype=torch.bool)))
+    compare_with_oracle(o, lse, ro, rl, torch.bfloat16, "ragged S")
+
+
+def test_out_of_range_metadata_is_clamped(gpu_device):
+    """kv_num_blocks beyond max_blocks and kv_indices beyond the last block are clamped."""
+    gen = torch.Generator().manual_seed(12)
+    S, D = 256, 64
+    q, k, v = (torch.randn(1, 1, S, D, generator=gen).to(torch.float16) for _ in range(3))
+    nb = torch.tensor([[[7, 2]]], dtype=torch.int32)            # max_blocks is 2
+    idx = torch.tensor([[[[0, 99], [-5, 1]]]], dtype=torch.int32)
+    tys = torch.full((1, 1, 2, 2), 2, dtype=torch.int32)
+    o, lse = run_kernel(q, k, v, nb, idx, tys, 128, 128, S, device=gpu_device)
+    nb2 = torch.tensor([[[2, 2]]], dtype=torch.int32)
+    idx2 = torch.tensor([[[[0, 1], [0, 1]]]], dtype=torch.int32)
+    o2, lse2 = run_kernel(q, k, v, nb2, idx2, tys, 128, 128, S, device=gpu_device)
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
+
+
+def test_non_default_stream(gpu_device):
+    w = make_workload("c1_causal", seed=2)
+    o_ref, lse_ref = run_workload(w, gpu_device)
+    s = torch.cuda.Stream(device=gpu_device)
+    with torch.cuda.stream(s):
+        o, lse = run_workload(w, gpu_device, stream=s.cuda_stream)
+    s.synchronize()
+    assert torch.equal(o, o_ref) and torch.equal(lse, lse_ref)
+
+
+def test_runs_are_bitwise_reproducible(gpu_device):
+    w = make_workload("c3_partial", seed=5, H=2, S=2048)
+    a = run_workload(w, gpu_device)
+    b = run_workload(w, gpu_device)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])

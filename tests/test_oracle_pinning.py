@@ -1,0 +1,166 @@
+"""Pins the CPU oracle (oracle/) before anything is compared against it.
+
+Each check is chosen so that a plausible mistake -- a dropped scale, softmax over the
+wrong axis, a transposed operand, block-local instead of global causal indices, a wrong
+empty-row convention -- fails at least one of them.  None of them retypes the oracle's
+own formula: they use a library routine, brute-force loops, closed forms, and the
+known answers the reference's generators printed (tests/golden/printed_masks.json).
+"""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import load_printed_masks, random_block_metadata, typed_pattern_to_metadata
+from oracle.block_walk import attention_block_walk
+from oracle.dense_oracle import (attention_dense_fp32, dense_mask_from_blocks, prefix_mask,
+                                 transfusion_mask_bruteforce)
+
+
+def _rand(gen, *shape):
+    return torch.randn(*shape, generator=gen)
+
+
+def test_dense_oracle_matches_library_sdpa():
+    gen = torch.Generator().manual_seed(1)
+    q, k, v = (_rand(gen, 2, 3, 96, 32) for _ in range(3))
+    mask = torch.rand(2, 3, 96, 96, generator=gen) < 0.5
+    mask[..., 0] = True  # the library returns NaN for empty rows; keep every row alive here
+    o, lse = attention_dense_fp32(q, k, v, mask)
+    ref = F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+    assert torch.allclose(o, ref, atol=2e-6, rtol=1e-5)
+    s = (q @ k.transpose(-1, -2)) / math.sqrt(32)
+    ref_lse = torch.logsumexp(s.masked_fill(~mask, float("-inf")), -1)
+    assert torch.allclose(lse, ref_lse, atol=1e-6)
+
+
+def test_dense_oracle_matches_bruteforce_loops():
+    gen = torch.Generator().manual_seed(2)
+    S, D = 7, 5
+    q, k, v = (_rand(gen, S, D).double() for _ in range(3))
+    mask = torch.rand(S, S, generator=gen) < 0.6
+    mask[3] = False  # an empty row
+    exp_o = torch.zeros(S, D, dtype=torch.float64)
+    exp_l = torch.full((S,), float("-inf"), dtype=torch.float64)
+    for i in range(S):
+        ws = []
+        for j in range(S):
+            if mask[i, j]:
+                dot = sum(q[i, d].item() * k[j, d].item() for d in range(D)) / math.sqrt(D)
+                ws.append((j, dot))
+        if not ws:
+            continue
+        z = sum(math.exp(w) for _, w in ws)
+        exp_l[i] = math.log(z)
+        for j, w in ws:
+            exp_o[i] += math.exp(w) / z * v[j]
+    o, lse = attention_dense_fp32(q, k, v, mask)
+    assert torch.allclose(o.double(), exp_o, atol=1e-6)
+    assert torch.equal(torch.isinf(lse), torch.isinf(exp_l))
+    live = ~torch.isinf(exp_l)
+    assert torch.allclose(lse.double()[live], exp_l[live], atol=1e-6)
+    assert (o[3] == 0).all() and lse[3] == float("-inf")
+
+
+def test_dense_oracle_closed_forms():
+    gen = torch.Generator().manual_seed(3)
+    S, D = 16, 8
+    v = _rand(gen, S, D)
+    # zero queries: uniform weights over the allowed keys -> mean of their V rows, lse = log n
+    q = torch.zeros(S, D)
+    k = _rand(gen, S, D)
+    causal = torch.tril(torch.ones(S, S, dtype=torch.bool))
+    o, lse = attention_dense_fp32(q, k, v, causal)
+    for i in range(S):
+        assert torch.allclose(o[i], v[: i + 1].mean(0), atol=1e-6)
+        assert abs(lse[i].item() - math.log(i + 1)) < 1e-6
+    # one allowed key: output is that V row exactly, lse = q.k / sqrt(D)
+    q = _rand(gen, S, D)
+    one = torch.zeros(S, S, dtype=torch.bool)
+    one[torch.arange(S), (torch.arange(S) * 5) % S] = True
+    o, lse = attention_dense_fp32(q, k, v, one)
+    cols = (torch.arange(S) * 5) % S
+    assert torch.allclose(o, v[cols], atol=1e-6)
+    assert torch.allclose(lse, (q * k[cols]).sum(-1) / math.sqrt(D), atol=1e-5)
+    # scale is 1/sqrt(D), not 1/D or 1: doubling D by zero-padding changes the result
+    # exactly as if the scores were divided by sqrt(2)
+    qp, kp = torch.cat([q, torch.zeros_like(q)], -1), torch.cat([k, torch.zeros_like(k)], -1)
+    o2, _ = attention_dense_fp32(qp, kp, v, causal)
+    o3, _ = attention_dense_fp32(q / math.sqrt(2.0), k, v, causal)
+    assert torch.allclose(o2, o3, atol=1e-6)
+
+
+def test_row_chunking_is_invisible():
+    gen = torch.Generator().manual_seed(4)
+    q, k, v = (_rand(gen, 2, 50, 16) for _ in range(3))
+    mask = torch.rand(2, 50, 50, generator=gen) < 0.4
+    a = attention_dense_fp32(q, k, v, mask, row_chunk=7)
+    b = attention_dense_fp32(q, k, v, mask, row_chunk=4096)
+    assert torch.allclose(a[0], b[0], atol=1e-6) and torch.equal(torch.isinf(a[1]), torch.isinf(b[1]))
+
+
+def test_transfusion_rule_prefix_form_matches_bruteforce():
+    from omni_attn_torch import modality_prefix_lengths, naive_attn_mask
+    S = 40
+    cases = [[], [(5, 10)], [(0, 7), (20, 6)], [(3, 4), (10, 25), (38, 2)], [(12, 0)]]
+    for spans in cases:
+        brute = transfusion_mask_bruteforce(S, spans)
+        mp = torch.zeros(1, max(1, len(spans)), 3, dtype=torch.long)
+        for m, (off, ln) in enumerate(spans):
+            mp[0, m] = torch.tensor([1, off, ln])
+        assert torch.equal(naive_attn_mask(S, mp)[0], brute), spans
+        assert torch.equal(prefix_mask(modality_prefix_lengths(mp, S), S)[0], brute), spans
+
+
+@pytest.mark.parametrize("pat", load_printed_masks()["typed_block_patterns"], ids=lambda p: p["source"])
+def test_block_semantics_against_printed_sparsity(pat):
+    """Typed block patterns + the sparsity the reference printed for their dense mask.
+    Patterns contain CAUSAL blocks off the diagonal, so block-local causal indices, or a
+    PARTIAL tile read transposed, change the number."""
+    S, QB, KB = pat["seq_len"], pat["Q_BLOCK_SIZE"], pat["KV_BLOCK_SIZE"]
+    nb, idx, tys, pidx, pm = typed_pattern_to_metadata(pat["rows"], True, QB, KB)
+    dense = dense_mask_from_blocks(nb, idx, tys, QB, KB, S, S, pidx, pm)
+    assert abs((1.0 - dense.float().mean().item()) - pat["sparsity"]) < 5e-5
+    # the C walk must realise the same mask: with q = 0 every allowed key has weight
+    # 1/n, so with V = one-hot(key) the output row is the mask row divided by n
+    q = torch.zeros(1, 1, S, 64)
+    k = torch.zeros(1, 1, S, 64)
+    for d0 in range(0, S, 64):
+        v = torch.zeros(1, 1, S, 64)
+        v[0, 0, d0:d0 + 64] = torch.eye(64)
+        o, lse = attention_block_walk(q, k, v, nb, idx, tys, QB, KB, S, pidx, pm)
+        n = dense[0, 0].sum(-1, keepdim=True).clamp(min=1).float()
+        assert torch.allclose(o[0, 0], dense[0, 0, :, d0:d0 + 64].float() / n, atol=1e-6)
+    assert torch.allclose(lse[0, 0], torch.log(dense[0, 0].sum(-1).float()), atol=1e-5)
+
+
+@pytest.mark.parametrize("QB,KB", [(128, 128), (128, 64), (64, 128), (64, 64)])
+def test_block_walk_matches_dense_oracle(QB, KB):
+    gen = torch.Generator().manual_seed(10 * QB + KB)
+    B, H, S, D = 2, 2, 512, 32
+    q, k, v = (_rand(gen, B, H, S, D) for _ in range(3))
+    nb, idx, tys, pidx, pm = random_block_metadata(gen, B, H, S // QB, S // KB, QB, KB, shuffle=True)
+    for seqlen in (S, S - 37):
+        dense = dense_mask_from_blocks(nb, idx, tys, QB, KB, S, S, pidx, pm, seqlen_orig=seqlen)
+        ro, rl = attention_dense_fp32(q, k, v, dense)
+        o, lse = attention_block_walk(q, k, v, nb, idx, tys, QB, KB, seqlen, pidx, pm)
+        assert torch.allclose(o, ro, atol=2e-5), (o - ro).abs().max()
+        assert torch.equal(torch.isinf(lse), torch.isinf(rl))
+        live = ~torch.isinf(rl)
+        assert torch.allclose(lse[live], rl[live], atol=2e-5)
+        assert (o[~live] == 0).all()
+        assert (~live).any(), "the case must contain empty rows"
+
+
+def test_bitless_partial_slot_is_skipped_by_the_walk():
+    """PARTIAL without stored bits contributes nothing (attn_naive.cu:119-131)."""
+    gen = torch.Generator().manual_seed(5)
+    q, k, v = (_rand(gen, 1, 1, 256, 32) for _ in range(3))
+    nb = torch.tensor([[[1, 2]]], dtype=torch.int32)
+    idx = torch.tensor([[[[0, 0], [0, 1]]]], dtype=torch.int32)
+    tys = torch.tensor([[[[1, 0], [3, 1]]]], dtype=torch.int32)
+    o, lse = attention_block_walk(q, k, v, nb, idx, tys, 128, 128, 256)
+    tys_skip = torch.tensor([[[[1, 0], [0, 1]]]], dtype=torch.int32)
+    o2, lse2 = attention_block_walk(q, k, v, nb, idx, tys_skip, 128, 128, 256)
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
