@@ -1,0 +1,169 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-sparse attention forward on one MI355X.
+
+One "step" is one forward launch over the whole synthetic batch of the workload, called
+through the C ABI with q/k/v and the block-mask metadata already resident in HBM.
+Prints ONE JSON line.  `value` is effective TFLOP/s: 4*QB*KB*D flops per listed
+(non-empty) block -- CAUSAL and PARTIAL blocks count as full tiles, softmax flops are
+not counted, EMPTY blocks count nothing -- divided by the wall time per step.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "omni-attention_amd")
+for _p in (ROOT, PKG):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+METRIC = "effective TFLOP/s (non-empty blocks) + % bf16 MFMA peak, 8K interleaved mask"
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs),
+# each scaled by the same counter's reading for a copy kernel of known size; None = not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def cpu_baseline(w, budget_s: float):
+    """The fp32 dense oracle timed on the host cores over a bounded sample of (b, h) slabs."""
+    import torch
+    from oracle.dense_oracle import attention_dense_fp32, prefix_mask
+
+    B, H, S, D = w.q.shape
+    m = w.block_mask
+    per_block = 4.0 * m.Q_BLOCK_SIZE * m.KV_BLOCK_SIZE * D
+    slabs = [(b, h) for h in range(H) for b in range(B)]
+    done, flops = 0, 0.0
+    t0 = time.perf_counter()
+    for b, h in slabs:
+        attention_dense_fp32(w.q[b, h], w.k[b, h], w.v[b, h], prefix_mask(w.prefix_len[b], S))
+        flops += per_block * float(m.kv_num_blocks[b, h].sum().item())
+        done += 1
+        if time.perf_counter() - t0 >= budget_s:
+            break
+    dt = time.perf_counter() - t0
+    return {
+        "value": flops / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{done} of {B * H} (batch, head) slabs of the same workload, dense fp32 "
+                  f"[S,S] scores per slab, {dt:.1f} s; effective flops of those slabs / time",
+        "ms_per_slab": dt / done * 1e3,
+    }
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2_interleaved")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-budget-s", type=float, default=12.0)
+    args = ap.parse_args(argv)
+    if args.gpus != 1:
+        print("bench.py measures one GPU: (batch, head) slabs are independent, so more GPUs would "
+              "only run disjoint slices of the same kernel; run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import omni_attn_capi
+    from baseline_configs import make_workload
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 1
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    omni_attn_capi.load_library()  # fail loudly when the HIP library is missing
+
+    w = make_workload(args.workload, seed=args.seed)
+    m = w.block_mask
+    B, H, S, D = w.q.shape
+    q, k, v = (t.to(dev) for t in (w.q, w.k, w.v))
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, S, dtype=torch.float32, device=dev)
+    nb, idx, tys = (t.to(dev) for t in (m.kv_num_blocks, m.kv_indices, m.block_mask_types))
+    pidx = None if m.partial_block_mask_indices is None else m.partial_block_mask_indices.to(dev)
+    pm = None if m.partial_block_masks is None else m.partial_block_masks.to(dev)
+    stream = torch.cuda.current_stream(dev)
+
+    def step():
+        omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, pidx, pm,
+                           stream=stream.cuda_stream)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    # timed region: exactly K steps, synchronised on both sides; events on the launch stream
+    # bracket every launch so that the kernel's own duration is measured in the same region
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        starts[i].record(stream)
+        step()
+        ends[i].record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    kernel_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
+    med_kernel_ms = statistics.median(kernel_ms)
+    ms_per_step = wall / args.steps * 1e3
+    flops = w.effective_flops
+    value = flops / (ms_per_step * 1e-3) / 1e12
+    achieved = flops / (avg_kernel_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": METRIC,
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": w.info["dtype"],
+        "data": "synthetic",
+        "config": {
+            "workload": f"{w.name}: B={B} H={H} S={S} D={D} {w.info['dtype']}, Q_BLOCK={m.Q_BLOCK_SIZE} "
+                        f"KV_BLOCK={m.KV_BLOCK_SIZE}, seed {args.seed}, image spans per batch element "
+                        f"{[len(s) for s in w.spans]}",
+            "nonempty_blocks": w.nonempty_blocks,
+            "total_blocks": B * H * m.num_q_blocks * m.num_kv_blocks,
+            "effective_gflop_per_step": flops / 1e9,
+        },
+        "pct_of_mfma_peak": 100.0 * value / MFMA_PEAK_TFLOPS,
+        "kernel_ms_median": med_kernel_ms,
+        "roofline": {
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / MFMA_PEAK_TFLOPS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "kernel_ms_avg": avg_kernel_ms,
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w, args.cpu_budget_s)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

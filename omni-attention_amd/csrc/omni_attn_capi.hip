@@ -41,7 +41,7 @@ extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v,
     return OMNI_ATTN_ERR_BAD_SHAPE;
   if (Tq != (S_pad + QB - 1) / QB) return OMNI_ATTN_ERR_BAD_SHAPE;
   const long long total = (long long)B * H * Tq;
-  if ((long long)S_pad * D > 0x7fffffffLL || total > 0x7fffffffLL - 8 ||
+  if ((long long)S_pad * D > 0x7fffffffLL || total > 0x7fffffffLL / 2 ||
       total * max_blocks > (1LL << 40))
     return OMNI_ATTN_ERR_TOO_LARGE;
 
@@ -62,8 +62,7 @@ extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v,
   p.Tk = (S_pad + KB - 1) / KB;
   p.max_blocks = max_blocks;
   p.seqlen = seqlen_orig < S_pad ? seqlen_orig : S_pad;
-  p.total_work = int(total);
-  p.work_per_xcd = int((total + 7) / 8);
+  p.n_slabs = B * H;
   p.sl2 = float(1.4426950408889634 / std::sqrt(double(D)));
 
   hipStream_t s = static_cast<hipStream_t>(stream);

@@ -15,9 +15,10 @@
 // per-lane scalar.
 //
 // A wave owns 32 query rows; a workgroup has QB/32 waves.  KV blocks are consumed in
-// steps of 64 keys (a 128-key block is two steps) from a double-buffered LDS tile
-// pair; the next step's K/V (and, for PARTIAL blocks, its mask bytes) are fetched
-// into registers while the current step computes.
+// steps of 64 keys (a 128-key block is two steps).  K and V tiles are double-buffered
+// in LDS and filled by direct global->LDS loads (no register staging); the K tile runs
+// one step ahead of the V tile so that S^T of step i+1 is issued to the matrix cores
+// before the softmax of step i runs on the vector ALU.  One workgroup barrier per step.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -52,8 +53,7 @@ struct FwdParams {
   int Tk;          // ceil(S / KB)
   int max_blocks;  // slots per query block
   int seqlen;      // min(seqlen_orig, S): rows/keys at or beyond it are padding
-  int total_work;  // B*H*Tq
-  int work_per_xcd;
+  int n_slabs;     // B*H
   float sl2;       // log2(e) / sqrt(D)
 };
 
@@ -89,17 +89,45 @@ __device__ __forceinline__ int k_swizzle(int row) {
   constexpr int C = D / 8;  // 16-byte chunks per row
   return (row / (16 / C)) % C;
 }
-// V is read with ds_read_b64_tr_b16: 4 lanes read 32 contiguous bytes of one row, the
-// next 4 lanes the next row.  The 32-byte unit index is XORed with the row.
+// V is read with ds_read_b64_tr_b16: within 16 lanes, 4 lanes read 32 contiguous bytes
+// of one row and the next 4 lanes the next row; lanes 16-31 read the neighbouring 32-byte
+// unit of the same 4 rows.  Bit 0 of the unit index (which half-wave group) is left
+// alone and the higher bits are XORed with the row, so the 32 lanes that are served
+// together touch 8 different 32-byte bank groups.
 template <int D>
 __device__ __forceinline__ int v_swizzle(int row) {
   constexpr int U = D / 16;  // 32-byte units per row
-  return (row / (8 / U)) % U;
+  if constexpr (U <= 2) return 0;
+  return 2 * ((row / (8 / U)) % (U / 2));
 }
 
 __device__ __forceinline__ s16x4_t lds_read_tr16(const uint16_t* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
       (__attribute__((address_space(3))) s16x4_t*)(p));
+}
+
+// Exchange between the lane pair (l, l ^ 32) without touching LDS: v_permlane32_swap
+// swaps the upper 32 lanes of its first operand with the lower 32 lanes of its second,
+// so with x in both operands one result holds {lo, lo} and the other {hi, hi}.
+// (The elements are copied to scalars before the bit cast: a bit cast applied directly
+// to a vector element expression reads element 0 for both.)
+__device__ __forceinline__ void pair_split(float x, float& lo, float& hi) {
+  typedef __attribute__((ext_vector_type(2))) unsigned u2;
+  const unsigned a = __builtin_bit_cast(unsigned, x);
+  const u2 r = __builtin_amdgcn_permlane32_swap(a, a, false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  lo = __builtin_bit_cast(float, r0);
+  hi = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ float pair_max(float x) {
+  float lo, hi;
+  pair_split(x, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  float lo, hi;
+  pair_split(x, lo, hi);
+  return lo + hi;
 }
 
 template <bool BF16, int D, int QB, int KB>
@@ -108,8 +136,50 @@ struct FwdTraits {
   static constexpr int kStep = 64;
   static constexpr int kTileElems = kStep * D;
   static constexpr size_t kLdsBytes =
-      size_t(2) * 2 * kTileElems * sizeof(uint16_t) + size_t(2) * QB * 2 * sizeof(uint32_t);
+      size_t(2) * 2 * kTileElems * sizeof(uint16_t) + size_t(QB) * 2 * sizeof(uint32_t);
 };
+
+// One step of the walk: 64 keys starting at row0, with the effective block mode.
+struct StepInfo {
+  int row0;
+  int mode;
+  int pid;
+};
+// The metadata words of a step as loaded; interpreted one iteration later so that no
+// instruction waits on a metadata load it has just issued.
+struct RawStep {
+  int kvb;
+  int ty;
+  int pid;
+};
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+// 16 bytes per lane from global memory straight into LDS: the wave's 64 chunks land at
+// lds_base + 16 * lane.  The global address is a wave-uniform 64-bit base plus a per-lane
+// 32-bit byte offset.  Written as inline asm so that the compiler does not order later
+// LDS reads of *other* buffers behind it with a vmcnt(0) wait; completion is waited for
+// explicitly (vmcnt(0) + workgroup barrier) before the filled buffer is read.
+__device__ __forceinline__ void global_to_lds_b128(const void* gbase_uniform, uint32_t byte_off,
+                                                   uint32_t lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds_base), "v"(byte_off), "s"(gbase_uniform)
+      : "memory", "m0");
+}
+// Block-mask metadata is read-only for the whole launch and every read of it is
+// wave-uniform: reading it through the constant address space makes these scalar loads
+// (SGPR results, no vector-memory latency in the instruction stream).
+__device__ __forceinline__ int32_t load_uniform(const int32_t* p) {
+  return *reinterpret_cast<const __attribute__((address_space(4))) int32_t*>(
+      reinterpret_cast<size_t>(p));
+}
+__device__ __forceinline__ uint32_t lds_offset_of(const void* p) {
+  return uint32_t(size_t((lds_void_t*)p));
+}
 
 template <bool BF16, int D, int QB, int KB>
 __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
@@ -118,26 +188,31 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   constexpr int STEP = Traits::kStep;
   constexpr int SPB = KB / STEP;        // steps per KV block
   constexpr int CPR = D / 8;            // 16-byte chunks per row
-  constexpr int NCH = STEP * CPR / NT;  // chunks per thread per tile
+  constexpr int NCH = STEP * CPR / NT;  // 16-byte chunks per thread per tile
   constexpr int KS = D / 16;            // MFMA k-steps of Q.K
   constexpr int DT = D / 32;            // 32-row tiles of O^T
   constexpr int TILE = Traits::kTileElems;
   static_assert(STEP * CPR % NT == 0, "tile must divide over the workgroup");
 
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-  uint16_t* sK = reinterpret_cast<uint16_t*>(lds_raw);  // [2][TILE]
-  uint16_t* sV = sK + 2 * TILE;                         // [2][TILE]
-  uint32_t* sBits = reinterpret_cast<uint32_t*>(sV + 2 * TILE);  // [2][QB*2]
+  uint16_t* sK = reinterpret_cast<uint16_t*>(lds_raw);           // [2][TILE]
+  uint16_t* sV = sK + 2 * TILE;                                  // [2][TILE]
+  uint32_t* sBits = reinterpret_cast<uint32_t*>(sV + 2 * TILE);  // [QB*2]
 
   // Workgroup -> (slab, query block).  Consecutive workgroup ids go round-robin over
-  // the 8 XCDs, so give each XCD one contiguous range of the work list: all query
-  // blocks of a (b,h) slab then share one XCD's L2 for that slab's K and V.  Inside a
-  // slab the last (longest, under causal masks) query block is issued first.
+  // the 8 XCDs.  XCD x takes the slabs bh with bh % 8 == x (every batch element's heads
+  // are spread over all XCDs, which balances batches with different masks), and walks
+  // them longest-first: query block Tq-1 of each of its slabs, then Tq-2, ...  The
+  // query blocks of one slab that run together walk the same K/V rows at about the
+  // same time, so that slab's K and V are served from the XCD's L2.
   const int wg = blockIdx.x;
-  const int work = (wg & 7) * p.work_per_xcd + (wg >> 3);
-  if (work >= p.total_work) return;
-  const int bh = work / p.Tq;
-  const int qb = p.Tq - 1 - (work - bh * p.Tq);
+  const int xcd = wg & 7;
+  const int slot = wg >> 3;
+  const int slabs_here = (p.n_slabs - xcd + 7) >> 3;
+  if (slot >= slabs_here * p.Tq) return;
+  const int qrank = slot / slabs_here;
+  const int bh = xcd + 8 * (slot - qrank * slabs_here);
+  const int qb = p.Tq - 1 - qrank;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -163,72 +238,128 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
 
   const size_t meta_row = size_t(bh) * p.Tq + qb;
   const size_t meta_off = meta_row * p.max_blocks;
-  int nb = p.kv_num_blocks[meta_row];
+  int nb = load_uniform(p.kv_num_blocks + meta_row);
   nb = nb < 0 ? 0 : (nb > p.max_blocks ? p.max_blocks : nb);
   const int nsteps = nb * SPB;
 
-  // Decode step `it` of the walk: first key row, effective mode, partial-mask index.
-  auto decode = [&](int it, int& kv_row0, int& mode, int& pid) {
-    const int j = it / SPB;
-    const int half = it - j * SPB;
-    int kvb = p.kv_indices[meta_off + j];
-    kvb = kvb < 0 ? 0 : (kvb >= p.Tk ? p.Tk - 1 : kvb);
-    const int ty = p.types[meta_off + j];
-    mode = (ty == kCausal || ty == kFull || ty == kPartial) ? ty : kMasked;
-    pid = -1;
-    if (ty == kPartial) {
-      if (p.partial_idx != nullptr && p.partial_masks != nullptr) pid = p.partial_idx[meta_off + j];
-      if (pid < 0) mode = kMasked;
+  // Metadata of step `it`: issue the (scalar) loads ...
+  const bool has_partial = p.partial_idx != nullptr && p.partial_masks != nullptr;
+  auto fetch_raw = [&](int it) {
+    RawStep r = {0, kMasked, -1};
+    if (it < nsteps) {
+      const int j = it / SPB;
+      r.kvb = load_uniform(p.kv_indices + meta_off + j);
+      r.ty = load_uniform(p.types + meta_off + j);
+      if (has_partial) r.pid = load_uniform(p.partial_idx + meta_off + j);
     }
-    kv_row0 = kvb * KB + half * STEP;
+    return r;
+  };
+  // ... and interpret them: first key row, effective mode, partial-mask index.
+  auto interpret = [&](int it, const RawStep& r) {
+    StepInfo si;
+    const int half = it % SPB;
+    const int kvb = r.kvb < 0 ? 0 : (r.kvb >= p.Tk ? p.Tk - 1 : r.kvb);
+    si.mode = (r.ty == kCausal || r.ty == kFull || r.ty == kPartial) ? r.ty : kMasked;
+    si.pid = r.pid;
+    if (r.ty == kPartial && r.pid < 0) si.mode = kMasked;
+    si.row0 = kvb * KB + half * STEP;
+    return si;
   };
 
-  u32x4_t kreg[NCH], vreg[NCH], mreg[2];
-
-  auto global_fetch = [&](int it, int kv_row0, int mode, int pid) {
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int x = tid + i * NT;
-      const int row = x / CPR;
-      const int ch = x % CPR;
-      int gr = kv_row0 + row;
-      gr = gr < p.S ? gr : p.S - 1;
-      const size_t off = size_t(gr) * D + ch * 8;
-      kreg[i] = *reinterpret_cast<const u32x4_t*>(gK + off);
-      vreg[i] = *reinterpret_cast<const u32x4_t*>(gV + off);
-    }
-    if (mode == kPartial) {
-      const int half = it % SPB;
-      const uint8_t* mp = p.partial_masks + size_t(pid) * (QB * KB) + size_t(tid >> 1) * KB +
-                          half * STEP + (tid & 1) * 32;
-      mreg[0] = *reinterpret_cast<const u32x4_t*>(mp);
-      mreg[1] = *reinterpret_cast<const u32x4_t*>(mp + 16);
-    }
+  // Direct global->LDS tile load: every lane fetches 16 bytes, the wave's 64 chunks land
+  // at consecutive LDS addresses: one wave-wide load fills 64 / CPR rows of the tile.
+  // The swizzle is applied on the global side: the lane that fills physical chunk
+  // (row, pch) fetches the logical chunk that belongs there.  The swizzle only depends
+  // on row modulo 16 (at most) and the loads of one thread are a multiple of 16 rows
+  // apart in every configuration except (QB=64, D=128), so one per-lane byte offset
+  // serves all loads of a thread and the rest of the address is wave-uniform.  A tile
+  // that would run past the last row of the slab clamps its rows instead.
+  constexpr int ROWS_PER_CALL = 64 / CPR;           // rows filled by one wave-wide load
+  constexpr int ROW_STRIDE = ROWS_PER_CALL * (NT / 64);  // rows between a thread's loads
+  constexpr bool kUniformSwizzle = ROW_STRIDE % 16 == 0;
+  const int ld_row = tid / CPR;  // row of this thread's first load
+  const int ld_pch = tid % CPR;
+  auto k_off = [&](int row) { return uint32_t(row * D + (ld_pch ^ k_swizzle<D>(row)) * 8) * 2u; };
+  auto v_off = [&](int row) {
+    return uint32_t(row * D + ((((ld_pch >> 1) ^ v_swizzle<D>(row)) << 1) | (ld_pch & 1)) * 8) * 2u;
   };
-
-  auto lds_commit = [&](int buf, int mode) {
-    uint16_t* dK = sK + buf * TILE;
-    uint16_t* dV = sV + buf * TILE;
+  const uint32_t koff0 = k_off(ld_row), voff0 = v_off(ld_row);
+  const uint32_t lds_k0 = lds_offset_of(sK) + uint32_t(w) * 1024u;
+  const uint32_t lds_v0 = lds_offset_of(sV) + uint32_t(w) * 1024u;
+  auto issue_tile = [&](const uint16_t* gsrc, bool is_v, uint32_t lds0, int buf, int kv_row0) {
+    const uint32_t dst = lds0 + uint32_t(buf) * (TILE * 2u);
+    const uint32_t off0 = is_v ? voff0 : koff0;
+    if (kv_row0 + STEP <= p.S) {
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int x = tid + i * NT;
-      const int row = x / CPR;
-      const int ch = x % CPR;
-      const int kch = ch ^ k_swizzle<D>(row);
-      const int vch = (((ch >> 1) ^ v_swizzle<D>(row)) << 1) | (ch & 1);
-      *reinterpret_cast<u32x4_t*>(dK + row * D + kch * 8) = kreg[i];
-      *reinterpret_cast<u32x4_t*>(dV + row * D + vch * 8) = vreg[i];
-    }
-    if (mode == kPartial) {
-      // 32 mask bytes (each 0 or 1) -> 32 bits; byte i of a dword lands in bit i.
-      uint32_t word = 0;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const uint32_t bytes = i < 4 ? mreg[0][i] : mreg[1][i - 4];
-        const uint32_t nib = ((bytes & 0x01010101u) * 0x01020408u) >> 24;
-        word |= nib << (4 * i);
+      for (int i = 0; i < NCH; ++i) {
+        uint32_t off = off0;
+        if constexpr (!kUniformSwizzle) {
+          const int row = ld_row + i * ROW_STRIDE;
+          off = (is_v ? v_off(row) : k_off(row)) - uint32_t(i * ROW_STRIDE * D * 2);
+        }
+        global_to_lds_b128(gsrc + size_t(kv_row0 + i * ROW_STRIDE) * D, off,
+                           dst + uint32_t(i) * (NT * 16u));
       }
-      sBits[buf * (QB * 2) + tid] = word;
+    } else {
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int row = ld_row + i * ROW_STRIDE;
+        int gr = kv_row0 + row;
+        gr = gr < p.S ? gr : p.S - 1;
+        const uint32_t off = (is_v ? v_off(row) : k_off(row)) - uint32_t(row * D * 2);
+        global_to_lds_b128(gsrc, off + uint32_t(gr) * (D * 2u), dst + uint32_t(i) * (NT * 16u));
+      }
+    }
+  };
+  auto issue_k = [&](int buf, int kv_row0) { issue_tile(gK, false, lds_k0, buf, kv_row0); };
+  auto issue_v = [&](int buf, int kv_row0) { issue_tile(gV, true, lds_v0, buf, kv_row0); };
+
+  // PARTIAL blocks: thread tid fetches 32 mask bytes of row tid/2 (a row of its own
+  // wave), packs them to 32 bits and parks the word in LDS for the two lanes that own
+  // the row.  Writer and readers are the same wave, so no workgroup barrier is needed.
+  // Done at the top of the step that needs it: no registers are held across steps for
+  // it, at the price of one exposed load latency per PARTIAL step.
+  auto stage_mask_bits = [&](int it, const StepInfo& si) {
+    const int half = it % SPB;
+    const uint8_t* mp = p.partial_masks + size_t(si.pid) * (QB * KB) + size_t(tid >> 1) * KB +
+                        half * STEP + (tid & 1) * 32;
+    const u32x4_t m0 = *reinterpret_cast<const u32x4_t*>(mp);
+    const u32x4_t m1 = *reinterpret_cast<const u32x4_t*>(mp + 16);
+    uint32_t word = 0;  // byte i (0 or 1) of the 32 -> bit i
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t bytes = i < 4 ? m0[i] : m1[i - 4];
+      const uint32_t nib = ((bytes & 0x01010101u) * 0x01020408u) >> 24;
+      word |= nib << (4 * i);
+    }
+    sBits[tid] = word;
+  };
+
+  // Wave-uniform classification of this wave's 32x64 tile of a step:
+  // 0 = nothing to do, 1 = no mask needed, 2 = masked path.
+  auto classify = [&](const StepInfo& si) {
+    if (si.mode == kMasked) return 0;
+    const bool clip = si.row0 + STEP > p.seqlen;
+    if (si.mode == kCausal) {
+      if (si.row0 > q_wave_min + 31) return 0;                       // all in the future
+      if (si.row0 + STEP - 1 <= q_wave_min && !clip) return 1;       // all in the past
+      return 2;
+    }
+    return (si.mode == kFull && !clip) ? 1 : 2;
+  };
+
+  // S^T = K . Q^T for the 64 keys of one LDS tile: two 32-key accumulator tiles.
+  auto qk_tile = [&](const uint16_t* tK, f32x16_t (&st)[2]) {
+    const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int row = 32 * t + c;
+        const int ch = (2 * s + g) ^ k_swizzle<D>(row);
+        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(tK + row * D + ch * 8);
+        st[t] = mfma_32x32x16<BF16>(a, qf[s], s == 0 ? zero : st[t]);
+      }
     }
   };
 
@@ -237,145 +368,151 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) ot[dt][r] = 0.f;
-  float m_run = -INFINITY;  // running row max, log2 domain (score * sl2)
+  float m_run = -INFINITY;  // reference point of the exponentials, log2 domain (score * sl2)
   float l_run = 0.f;        // this lane's share of the running row sum
 
-  int cur_row0 = 0, cur_mode = kMasked, cur_pid = -1;
-  if (nsteps > 0) {
-    decode(0, cur_row0, cur_mode, cur_pid);
-    global_fetch(0, cur_row0, cur_mode, cur_pid);
-    lds_commit(0, cur_mode);
-  }
-  __syncthreads();
-
-  for (int it = 0; it < nsteps; ++it) {
-    const int buf = it & 1;
-    int nxt_row0 = 0, nxt_mode = kMasked, nxt_pid = -1;
-    const bool has_next = it + 1 < nsteps;
-    if (has_next) {
-      decode(it + 1, nxt_row0, nxt_mode, nxt_pid);
-      global_fetch(it + 1, nxt_row0, nxt_mode, nxt_pid);
-    }
-
-    // Wave-uniform classification of this wave's 32x64 tile.
-    const bool clip = cur_row0 + STEP > p.seqlen;
-    bool skip = cur_mode == kMasked;
-    bool masked_path = cur_mode != kFull || clip;
-    if (cur_mode == kCausal) {
-      if (cur_row0 > q_wave_min + 31) skip = true;                      // all in the future
-      else if (cur_row0 + STEP - 1 <= q_wave_min && !clip) masked_path = false;  // all in the past
-    }
-
-    if (!skip) {
-      const uint16_t* tK = sK + buf * TILE;
-      const uint16_t* tV = sV + buf * TILE;
-
-      // S^T = K . Q^T : two 32-key tiles.
-      f32x16_t st[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) st[t][r] = 0.f;
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const int row = 32 * t + c;
-          const int ch = (2 * s + g) ^ k_swizzle<D>(row);
-          const u32x4_t a = *reinterpret_cast<const u32x4_t*>(tK + row * D + ch * 8);
-          st[t] = mfma_32x32x16<BF16>(a, qf[s], st[t]);
-        }
+  // Mask (if needed) + online softmax of one step; leaves P (fp32) in st.
+  auto softmax_step = [&](f32x16_t (&st)[2], const StepInfo& si, bool masked_path) {
+    if (masked_path) {
+      // Register r of tile t holds key  row0 + 32t + 8(r/4) + 4g + r%4.
+      int limit = p.seqlen - 1;
+      if (si.mode == kCausal) limit = limit < q_row ? limit : q_row;
+      const int lim_l = limit - si.row0 - 4 * g;
+      uint32_t kw0 = 0xffffffffu, kw1 = 0xffffffffu;
+      if (si.mode == kPartial) {
+        const u32x2_t bw = *reinterpret_cast<const u32x2_t*>(sBits + (32 * w + c) * 2);
+        kw0 = bw[0];
+        kw1 = bw[1];
       }
-
-      if (masked_path) {
-        // Register r of tile t holds key  cur_row0 + 32t + 8(r/4) + 4g + r%4.
-        int limit = p.seqlen - 1;
-        if (cur_mode == kCausal) limit = limit < q_row ? limit : q_row;
-        const int lim_l = limit - cur_row0 - 4 * g;
-        uint32_t kw0 = 0xffffffffu, kw1 = 0xffffffffu;
-        if (cur_mode == kPartial) {
-          const u32x2_t bw = *reinterpret_cast<const u32x2_t*>(sBits + buf * (QB * 2) + (32 * w + c) * 2);
-          kw0 = bw[0];
-          kw1 = bw[1];
-        }
-        kw0 >>= 4 * g;
-        kw1 >>= 4 * g;
+      kw0 >>= 4 * g;
+      kw1 >>= 4 * g;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const uint32_t kw = t == 0 ? kw0 : kw1;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int kl = 8 * (r >> 2) + (r & 3);
-            const bool keep = (32 * t + kl <= lim_l) && ((kw >> kl) & 1u);
-            st[t][r] = keep ? st[t][r] : -INFINITY;
-          }
-        }
-      }
-
-      // Online softmax (log2 domain).  The row lives in lanes c and c+32.
-      float mx = st[0][0];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[t][r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m_run, mx * p.sl2);
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
-      m_run = m_new;
-      float rs = 0.f;
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t) {
+        const uint32_t kw = t == 0 ? kw0 : kw1;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(st[t][r], p.sl2, -m_safe));
-          st[t][r] = pv;
-          rs += pv;
+          const int kl = 8 * (r >> 2) + (r & 3);
+          const bool keep = (32 * t + kl <= lim_l) && ((kw >> kl) & 1u);
+          st[t][r] = keep ? st[t][r] : -INFINITY;
         }
-      l_run = l_run * alpha + rs;
+      }
+    }
+    // The row lives in lanes c and c+32.
+    float mx = st[0][0];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[t][r]);
+    mx = pair_max(mx);
+    // The reference point m_run of the exponentials only has to stay within 2^kSlack of
+    // the true running max (P then stays below 2^kSlack, exact in fp32 and well inside
+    // the 16-bit types' range), so it is moved -- and O, l rescaled -- only when some
+    // row of the wave outgrows it by more than that.  The decision is wave-uniform; the
+    // result is the same sum with a different common factor.
+    constexpr float kSlack = 6.f;
+    const float m_cand = mx * p.sl2;
+    if (__builtin_amdgcn_ballot_w64(m_cand > m_run + kSlack) != 0) {
+      const float m_new = fmaxf(m_run, m_cand);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);  // m_run = -inf -> 0
+      m_run = m_new;
+      l_run *= alpha;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) ot[dt][r] *= alpha;
+    }
+    const float m_ref = m_run == -INFINITY ? 0.f : m_run;
+    float rs = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(st[t][r], p.sl2, -m_ref));
+        st[t][r] = pv;
+        rs += pv;
+      }
+    l_run += rs;
+  };
 
-      // O^T += V^T . P^T.  k-slot e of lane group g in k-step (t, s2) is key
-      // 32t + 16 s2 + 8(e/4) + 4g + e%4 -- the accumulator order of S^T.
+  // O^T += V^T . P^T.  k-slot e of lane group g in k-step (t, s2) is key
+  // 32t + 16 s2 + 8(e/4) + 4g + e%4 -- the accumulator order of S^T.
+  auto pv_tile = [&](const uint16_t* tV, const f32x16_t (&st)[2]) {
+    const int i16 = c & 15;
+    const int j16 = c >> 4;
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < 2; ++t) {
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          u32x4_t pb;
+      for (int s2 = 0; s2 < 2; ++s2) {
+        u32x4_t pb;
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            pb[e] = pack2<BF16>(st[t][8 * s2 + 2 * e], st[t][8 * s2 + 2 * e + 1]);
-          const int i16 = c & 15;
-          const int j16 = c >> 4;
-          const int vrow = 32 * t + 16 * s2 + 4 * g + (i16 >> 2);
+        for (int e = 0; e < 4; ++e)
+          pb[e] = pack2<BF16>(st[t][8 * s2 + 2 * e], st[t][8 * s2 + 2 * e + 1]);
+        const int vrow = 32 * t + 16 * s2 + 4 * g + (i16 >> 2);
 #pragma unroll
-          for (int dt = 0; dt < DT; ++dt) {
-            const int unit = 2 * dt + j16;
-            const int u0 = unit ^ v_swizzle<D>(vrow);
-            const int u1 = unit ^ v_swizzle<D>(vrow + 8);
-            const s16x4_t lo = lds_read_tr16(tV + vrow * D + u0 * 16 + (i16 & 3) * 4);
-            const s16x4_t hi = lds_read_tr16(tV + (vrow + 8) * D + u1 * 16 + (i16 & 3) * 4);
-            const u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo);
-            const u32x2_t hi2 = __builtin_bit_cast(u32x2_t, hi);
-            const u32x4_t a = {lo2[0], lo2[1], hi2[0], hi2[1]};
-            ot[dt] = mfma_32x32x16<BF16>(a, pb, ot[dt]);
-          }
+        for (int dt = 0; dt < DT; ++dt) {
+          const int unit = 2 * dt + j16;
+          const int u0 = unit ^ v_swizzle<D>(vrow);
+          const int u1 = unit ^ v_swizzle<D>(vrow + 8);
+          const s16x4_t lo = lds_read_tr16(tV + vrow * D + u0 * 16 + (i16 & 3) * 4);
+          const s16x4_t hi = lds_read_tr16(tV + (vrow + 8) * D + u1 * 16 + (i16 & 3) * 4);
+          const u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo);
+          const u32x2_t hi2 = __builtin_bit_cast(u32x2_t, hi);
+          const u32x4_t a = {lo2[0], lo2[1], hi2[0], hi2[1]};
+          ot[dt] = mfma_32x32x16<BF16>(a, pb, ot[dt]);
         }
       }
     }
+  };
 
-    if (has_next) lds_commit(buf ^ 1, nxt_mode);
+  // ---- software pipeline ----------------------------------------------------------
+  // Top of iteration `it` (before the barrier): in flight are K(it+1) -> sK[(it+1)&1] and
+  // V(it) -> sV[it&1]; st_cur holds S^T of step it.  After the barrier every wave has
+  // finished reading sK[it&1] (S^T of step it) and sV[(it-1)&1] (PV of step it-1), so
+  // those two buffers are refilled with K(it+2) and V(it+1).
+  // Step descriptors: raw metadata words are loaded three steps ahead and interpreted
+  // one iteration later, two steps ahead of their first use (the K tile load).
+  StepInfo cur = interpret(0, fetch_raw(0));
+  StepInfo nxt = interpret(1, fetch_raw(1));
+  StepInfo nn = interpret(2, fetch_raw(2));
+  RawStep raw3 = fetch_raw(3);
+  int cls_cur = classify(cur), cls_nxt = nsteps > 1 ? classify(nxt) : 0;
+  f32x16_t st_cur[2], st_nxt[2];
+  if (nsteps > 0) {
+    issue_k(0, cur.row0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
-    cur_row0 = nxt_row0;
-    cur_mode = nxt_mode;
-    cur_pid = nxt_pid;
+    if (nsteps > 1) issue_k(1, nxt.row0);
+    issue_v(0, cur.row0);
+    if (cls_cur != 0) qk_tile(sK, st_cur);
+  }
+
+  for (int it = 0; it < nsteps; ++it) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's tile loads have landed
+    __syncthreads();
+    if (it + 2 < nsteps) issue_k(it & 1, nn.row0);
+    if (it + 1 < nsteps) issue_v((it + 1) & 1, nxt.row0);
+    const StepInfo n3 = interpret(it + 3, raw3);
+    raw3 = fetch_raw(it + 4);
+    if (cur.mode == kPartial) stage_mask_bits(it, cur);
+
+    if (cls_nxt != 0) qk_tile(sK + ((it + 1) & 1) * TILE, st_nxt);
+    if (cls_cur != 0) {
+      softmax_step(st_cur, cur, cls_cur == 2);
+      pv_tile(sV + (it & 1) * TILE, st_cur);
+    }
+
+#pragma unroll
+    for (int t = 0; t < 2; ++t) st_cur[t] = st_nxt[t];
+    cur = nxt;
+    cls_cur = cls_nxt;
+    nxt = nn;
+    cls_nxt = (it + 2 < nsteps) ? classify(nn) : 0;
+    nn = n3;
   }
 
   // Epilogue: O = O^T / l, zeros for rows without any allowed key or beyond seqlen.
-  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float l_tot = pair_sum(l_run);
   const bool live = (q_row < p.seqlen) && (l_tot > 0.f);
   const float inv = live ? 1.f / l_tot : 0.f;
   if (q_row < p.S) {
@@ -406,7 +543,8 @@ int launch_fwd(const FwdParams& p, hipStream_t stream) {
                                      hipFuncAttributeMaxDynamicSharedMemorySize,
                                      int(Traits::kLdsBytes));
   if (e != hipSuccess) return int(e);
-  const dim3 grid(unsigned(p.work_per_xcd) * 8u);
+  const unsigned slabs_per_xcd = unsigned(p.n_slabs + 7) / 8u;
+  const dim3 grid(8u * slabs_per_xcd * unsigned(p.Tq));
   const dim3 block(Traits::kThreads);
   hipLaunchKernelGGL(kern, grid, block, Traits::kLdsBytes, stream, p);
   return int(hipGetLastError());
