@@ -27,7 +27,10 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs),
 # each scaled by the same counter's reading for a copy kernel of known size; None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # FETCH_SIZE 126003 KiB x 2.0 (the 256 MiB copy reads 131088) + WRITE_SIZE 66583 KiB x 1.0
+    "c2_interleaved": int((126003 * 2.0 + 66583) * 1024),
+}
 
 
 def cpu_baseline(w, budget_s: float):
@@ -68,6 +71,9 @@ def main(argv=None):
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget-s", type=float, default=12.0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy, so that a counter run of this "
+                         "command shows what FETCH_SIZE / WRITE_SIZE read for a known traffic")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py measures one GPU: (batch, head) slabs are independent, so more GPUs would "
@@ -117,6 +123,12 @@ def main(argv=None):
         ends[i].record(stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+
+    if args.calibrate_copy:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
 
     kernel_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
     avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)

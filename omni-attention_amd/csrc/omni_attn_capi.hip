@@ -63,6 +63,10 @@ extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v,
   p.max_blocks = max_blocks;
   p.seqlen = seqlen_orig < S_pad ? seqlen_orig : S_pad;
   p.n_slabs = B * H;
+  // An XCD has 32 CUs and a CU holds two workgroups of this kernel (a Q_BLOCK 64
+  // workgroup is half the size, four fit).
+  const int slots_per_xcd = 32 * (QB == 128 ? 2 : 4);
+  p.slab_group = slots_per_xcd / Tq > 1 ? slots_per_xcd / Tq : 1;
   p.sl2 = float(1.4426950408889634 / std::sqrt(double(D)));
 
   hipStream_t s = static_cast<hipStream_t>(stream);

@@ -54,6 +54,7 @@ struct FwdParams {
   int max_blocks;  // slots per query block
   int seqlen;      // min(seqlen_orig, S): rows/keys at or beyond it are padding
   int n_slabs;     // B*H
+  int slab_group;  // slabs of one XCD that are walked together (>= 1)
   float sl2;       // log2(e) / sqrt(D)
 };
 
@@ -201,17 +202,25 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
 
   // Workgroup -> (slab, query block).  Consecutive workgroup ids go round-robin over
   // the 8 XCDs.  XCD x takes the slabs bh with bh % 8 == x (every batch element's heads
-  // are spread over all XCDs, which balances batches with different masks), and walks
-  // them longest-first: query block Tq-1 of each of its slabs, then Tq-2, ...  The
-  // query blocks of one slab that run together walk the same K/V rows at about the
-  // same time, so that slab's K and V are served from the XCD's L2.
+  // are spread over all XCDs, which balances batches with different masks) and works
+  // through them in groups of p.slab_group slabs, sized so that one group's query
+  // blocks just fill the XCD's workgroup slots: the workgroups that run together then
+  // belong to one or two slabs and walk the same K/V rows at about the same time, so
+  // each K/V tile is fetched from HBM once and served from the XCD's L2 to the other
+  // query blocks.  Inside a group the order is longest-first: query block Tq-1 of each
+  // slab of the group, then Tq-2, ...
   const int wg = blockIdx.x;
   const int xcd = wg & 7;
   const int slot = wg >> 3;
   const int slabs_here = (p.n_slabs - xcd + 7) >> 3;
   if (slot >= slabs_here * p.Tq) return;
-  const int qrank = slot / slabs_here;
-  const int bh = xcd + 8 * (slot - qrank * slabs_here);
+  const int per_group = p.slab_group * p.Tq;
+  const int gi = slot / per_group;
+  const int in_group = slot - gi * per_group;
+  const int g_left = slabs_here - gi * p.slab_group;
+  const int g_eff = g_left < p.slab_group ? g_left : p.slab_group;
+  const int qrank = in_group / g_eff;
+  const int bh = xcd + 8 * (gi * p.slab_group + (in_group - qrank * g_eff));
   const int qb = p.Tq - 1 - qrank;
 
   const int tid = threadIdx.x;
