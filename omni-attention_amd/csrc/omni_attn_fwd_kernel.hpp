@@ -16,13 +16,27 @@
 //
 // A wave owns 32 query rows; a workgroup has QB/32 waves.  KV blocks are consumed in
 // steps of 64 keys (a 128-key block is two steps).  K and V tiles are double-buffered
-// in LDS and filled by direct global->LDS loads (no register staging); the K tile runs
-// one step ahead of the V tile so that S^T of step i+1 is issued to the matrix cores
-// before the softmax of step i runs on the vector ALU.  One workgroup barrier per step.
+// in LDS and filled by direct buffer->LDS loads (no register staging, out-of-range rows
+// read as zeros).
+//
+// The walk is software-pipelined so that the matrix cores and the vector ALU work on
+// different steps inside ONE instruction stream: iteration i of a wave issues the 2*D/16
+// MFMAs of S^T(i+1) and the D/8 MFMAs of O^T += V^T.P^T(i-1) while its vector
+// instructions do the online softmax of step i.  None of the three depends on another
+// inside the iteration, and the source spells the interleaving out: the iteration is a
+// sequence of slots, each with one MFMA, the LDS fetch of the operand four slots ahead, a
+// share of the softmax and -- in the early slots -- one tile load, with a scheduling fence
+// after every slot.  (A wave that issues MFMAs back to back leaves other waves of its
+// SIMD almost no vector issue slots; vector instructions placed between the MFMAs of the
+// same wave are nearly free.)  Two iterations are unrolled so that the accumulators of
+// S^T and the packed P alternate between two register sets without copies.
+// One workgroup barrier per step.
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <utility>
 
 namespace omni_attn {
 
@@ -146,29 +160,43 @@ struct StepInfo {
   int mode;
   int pid;
 };
-// The metadata words of a step as loaded; interpreted one iteration later so that no
-// instruction waits on a metadata load it has just issued.
-struct RawStep {
-  int kvb;
-  int ty;
-  int pid;
-};
 
 typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((ext_vector_type(4))) int32_t i32x4_t;
 
-// 16 bytes per lane from global memory straight into LDS: the wave's 64 chunks land at
-// lds_base + 16 * lane.  The global address is a wave-uniform 64-bit base plus a per-lane
-// 32-bit byte offset.  Written as inline asm so that the compiler does not order later
-// LDS reads of *other* buffers behind it with a vmcnt(0) wait; completion is waited for
-// explicitly (vmcnt(0) + workgroup barrier) before the filled buffer is read.
-__device__ __forceinline__ void global_to_lds_b128(const void* gbase_uniform, uint32_t byte_off,
-                                                   uint32_t lds_base) {
+// Buffer resource for a slab of `bytes` bytes: raw (unstructured) addressing, so a lane
+// whose byte offset is at or beyond `bytes` reads zeros instead of faulting.
+__device__ __forceinline__ i32x4_t make_buffer_resource(const void* base, uint32_t bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(base);
+  i32x4_t r;
+  r[0] = __builtin_amdgcn_readfirstlane(int32_t(uint32_t(a)));
+  r[1] = __builtin_amdgcn_readfirstlane(int32_t(uint32_t(a >> 32) & 0xffffu));
+  r[2] = __builtin_amdgcn_readfirstlane(int32_t(bytes));
+  r[3] = 0x00020000;
+  return r;
+}
+// 16 bytes per lane from a buffer straight into LDS: the wave's 64 chunks land at
+// lds_base + 16 * lane.  The source offset is a wave-uniform part plus a per-lane part.
+// Written as inline asm so that the compiler does not order later LDS reads of *other*
+// buffers behind it with a vmcnt(0) wait; completion is waited for explicitly (vmcnt(0) +
+// workgroup barrier) before the filled buffer is read.
+__device__ __forceinline__ void buffer_to_lds_b128(i32x4_t rsrc, uint32_t lane_off,
+                                                   uint32_t uniform_off, uint32_t lds_base) {
+  // (Every scalar operand goes through readfirstlane: that is free for a value that is
+  // already in scalar registers and keeps the operand legal if the compiler has chosen
+  // to compute a uniform value with vector instructions.)
+  i32x4_t r;
+  r[0] = __builtin_amdgcn_readfirstlane(rsrc[0]);
+  r[1] = __builtin_amdgcn_readfirstlane(rsrc[1]);
+  r[2] = __builtin_amdgcn_readfirstlane(rsrc[2]);
+  r[3] = __builtin_amdgcn_readfirstlane(rsrc[3]);
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
       "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %1, %2"
+      "buffer_load_dwordx4 %1, %2, %3 offen lds"
       :
-      : "s"(lds_base), "v"(byte_off), "s"(gbase_uniform)
+      : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(lane_off), "s"(r),
+        "s"(__builtin_amdgcn_readfirstlane(uniform_off))
       : "memory", "m0");
 }
 // Block-mask metadata is read-only for the whole launch and every read of it is
@@ -180,6 +208,28 @@ __device__ __forceinline__ int32_t load_uniform(const int32_t* p) {
 }
 __device__ __forceinline__ uint32_t lds_offset_of(const void* p) {
   return uint32_t(size_t((lds_void_t*)p));
+}
+
+// An empty asm that "modifies" its operands: the values have to be computed before
+// this point of the instruction stream (the optimizer would otherwise sink work whose
+// results are only needed much later out of the place it was written in).
+__device__ __forceinline__ void pin(float& a) { asm volatile("" : "+v"(a)); }
+__device__ __forceinline__ void pin(uint32_t& a) { asm volatile("" : "+v"(a)); }
+__device__ __forceinline__ void pin(float& a, float& b) { asm volatile("" : "+v"(a), "+v"(b)); }
+
+template <int V>
+struct IntC {
+  static constexpr int value = V;
+};
+// f(IntC<0>{}), f(IntC<1>{}), ... f(IntC<N-1>{}): a loop whose index is a compile-time
+// constant inside the body (register arrays indexed with it never go to scratch memory).
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(IntC<Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 template <bool BF16, int D, int QB, int KB>
@@ -230,8 +280,9 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   const int c = lane & 31;
 
   const size_t slab = size_t(bh) * size_t(p.S) * D;
-  const uint16_t* __restrict__ gK = p.k + slab;
-  const uint16_t* __restrict__ gV = p.v + slab;
+  const uint32_t slab_bytes = uint32_t(p.S) * uint32_t(D * 2);
+  const i32x4_t rK = make_buffer_resource(p.k + slab, slab_bytes);
+  const i32x4_t rV = make_buffer_resource(p.v + slab, slab_bytes);
 
   const int q_row = qb * QB + 32 * w + c;  // this lane's query row inside the slab
   const int q_wave_min = qb * QB + 32 * w;
@@ -251,83 +302,80 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   nb = nb < 0 ? 0 : (nb > p.max_blocks ? p.max_blocks : nb);
   const int nsteps = nb * SPB;
 
-  // Metadata of step `it`: issue the (scalar) loads ...
+  // Block metadata lives in registers: lane i of every wave holds the three words of
+  // block 64 * chunk + i of this query block's list, and a step's words are picked out
+  // with v_readlane -- no memory instruction per step.  A new chunk is fetched when the
+  // walk reaches it (every 64 blocks).
   const bool has_partial = p.partial_idx != nullptr && p.partial_masks != nullptr;
-  auto fetch_raw = [&](int it) {
-    RawStep r = {0, kMasked, -1};
-    if (it < nsteps) {
-      const int j = it / SPB;
-      r.kvb = load_uniform(p.kv_indices + meta_off + j);
-      r.ty = load_uniform(p.types + meta_off + j);
-      if (has_partial) r.pid = load_uniform(p.partial_idx + meta_off + j);
-    }
-    return r;
+  int32_t mv_kvb = 0, mv_ty = kMasked, mv_pid = -1;
+  auto load_chunk = [&](int chunk) {
+    const int j = chunk * 64 + lane;
+    const bool ok = j < nb;
+    const size_t o = meta_off + size_t(ok ? j : 0);
+    const int32_t kvb = p.kv_indices[o];
+    const int32_t ty = p.types[o];
+    const int32_t pid = has_partial ? p.partial_idx[o] : -1;
+    mv_kvb = ok ? kvb : 0;
+    mv_ty = ok ? ty : int32_t(kMasked);
+    mv_pid = ok ? pid : -1;
   };
-  // ... and interpret them: first key row, effective mode, partial-mask index.
-  auto interpret = [&](int it, const RawStep& r) {
+  // Step `it` (clamped to the last step of the walk; steps past the end are only ever
+  // used as the address of a tile load whose data nobody reads).
+  auto step_info = [&](int it) {
+    const int itc = it < nsteps ? it : nsteps - 1;
+    const int j = itc / SPB;
+    if (itc == it && itc % SPB == 0 && (j & 63) == 0 && j > 0) load_chunk(j >> 6);
+    const int ln = j & 63;
+    const int kvb_raw = __builtin_amdgcn_readlane(mv_kvb, ln);
+    const int ty = __builtin_amdgcn_readlane(mv_ty, ln);
+    const int pid = __builtin_amdgcn_readlane(mv_pid, ln);
     StepInfo si;
-    const int half = it % SPB;
-    const int kvb = r.kvb < 0 ? 0 : (r.kvb >= p.Tk ? p.Tk - 1 : r.kvb);
-    si.mode = (r.ty == kCausal || r.ty == kFull || r.ty == kPartial) ? r.ty : kMasked;
-    si.pid = r.pid;
-    if (r.ty == kPartial && r.pid < 0) si.mode = kMasked;
-    si.row0 = kvb * KB + half * STEP;
+    const int kvb = kvb_raw < 0 ? 0 : (kvb_raw >= p.Tk ? p.Tk - 1 : kvb_raw);
+    si.mode = (ty == kCausal || ty == kFull || ty == kPartial) ? ty : kMasked;
+    si.pid = pid;
+    if (ty == kPartial && pid < 0) si.mode = kMasked;
+    si.row0 = kvb * KB + (itc % SPB) * STEP;
     return si;
   };
 
-  // Direct global->LDS tile load: every lane fetches 16 bytes, the wave's 64 chunks land
+  // Direct buffer->LDS tile load: every lane fetches 16 bytes, the wave's 64 chunks land
   // at consecutive LDS addresses: one wave-wide load fills 64 / CPR rows of the tile.
-  // The swizzle is applied on the global side: the lane that fills physical chunk
-  // (row, pch) fetches the logical chunk that belongs there.  The swizzle only depends
-  // on row modulo 16 (at most) and the loads of one thread are a multiple of 16 rows
-  // apart in every configuration except (QB=64, D=128), so one per-lane byte offset
-  // serves all loads of a thread and the rest of the address is wave-uniform.  A tile
-  // that would run past the last row of the slab clamps its rows instead.
-  constexpr int ROWS_PER_CALL = 64 / CPR;           // rows filled by one wave-wide load
+  // The swizzle is applied on the source side: the lane that fills physical chunk
+  // (row, pch) fetches the logical chunk that belongs there.  The swizzle depends on the
+  // row modulo 16 at most and a thread's loads are ROW_STRIDE rows apart, so one or two
+  // per-lane byte offsets serve all loads of a thread; the rest of the address is
+  // wave-uniform and goes through the scalar offset of the load.
+  constexpr int ROWS_PER_CALL = 64 / CPR;                // rows filled by one wave-wide load
   constexpr int ROW_STRIDE = ROWS_PER_CALL * (NT / 64);  // rows between a thread's loads
-  constexpr bool kUniformSwizzle = ROW_STRIDE % 16 == 0;
+  constexpr int KPER = ROW_STRIDE % 16 == 0 ? 1 : 2;     // distinct K lane offsets
+  static_assert((KPER * ROW_STRIDE) % 16 == 0, "K swizzle must repeat over a thread's loads");
+  static_assert(ROW_STRIDE % 8 == 0, "V swizzle must be the same for all loads of a thread");
   const int ld_row = tid / CPR;  // row of this thread's first load
   const int ld_pch = tid % CPR;
   auto k_off = [&](int row) { return uint32_t(row * D + (ld_pch ^ k_swizzle<D>(row)) * 8) * 2u; };
   auto v_off = [&](int row) {
     return uint32_t(row * D + ((((ld_pch >> 1) ^ v_swizzle<D>(row)) << 1) | (ld_pch & 1)) * 8) * 2u;
   };
-  const uint32_t koff0 = k_off(ld_row), voff0 = v_off(ld_row);
+  uint32_t koff[KPER];
+#pragma unroll
+  for (int i = 0; i < KPER; ++i)
+    koff[i] = k_off(ld_row + i * ROW_STRIDE) - uint32_t(i * ROW_STRIDE * D * 2);
+  const uint32_t voff = v_off(ld_row);
   const uint32_t lds_k0 = lds_offset_of(sK) + uint32_t(w) * 1024u;
   const uint32_t lds_v0 = lds_offset_of(sV) + uint32_t(w) * 1024u;
-  auto issue_tile = [&](const uint16_t* gsrc, bool is_v, uint32_t lds0, int buf, int kv_row0) {
-    const uint32_t dst = lds0 + uint32_t(buf) * (TILE * 2u);
-    const uint32_t off0 = is_v ? voff0 : koff0;
-    if (kv_row0 + STEP <= p.S) {
-#pragma unroll
-      for (int i = 0; i < NCH; ++i) {
-        uint32_t off = off0;
-        if constexpr (!kUniformSwizzle) {
-          const int row = ld_row + i * ROW_STRIDE;
-          off = (is_v ? v_off(row) : k_off(row)) - uint32_t(i * ROW_STRIDE * D * 2);
-        }
-        global_to_lds_b128(gsrc + size_t(kv_row0 + i * ROW_STRIDE) * D, off,
-                           dst + uint32_t(i) * (NT * 16u));
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < NCH; ++i) {
-        const int row = ld_row + i * ROW_STRIDE;
-        int gr = kv_row0 + row;
-        gr = gr < p.S ? gr : p.S - 1;
-        const uint32_t off = (is_v ? v_off(row) : k_off(row)) - uint32_t(row * D * 2);
-        global_to_lds_b128(gsrc, off + uint32_t(gr) * (D * 2u), dst + uint32_t(i) * (NT * 16u));
-      }
-    }
+  // Load number n of a tile pair: n < NCH is part n of the V tile, the rest the K tile.
+  auto issue_load = [&](int n, int buf, int k_row0, int v_row0) {
+    const bool is_v = n < NCH;
+    const int i = is_v ? n : n - NCH;
+    const uint32_t dst = (is_v ? lds_v0 : lds_k0) + uint32_t(buf) * (TILE * 2u) + uint32_t(i) * (NT * 16u);
+    const uint32_t row = uint32_t(is_v ? v_row0 : k_row0) + uint32_t(i * ROW_STRIDE);
+    buffer_to_lds_b128(is_v ? rV : rK, is_v ? voff : koff[i % KPER], row * uint32_t(D * 2), dst);
   };
-  auto issue_k = [&](int buf, int kv_row0) { issue_tile(gK, false, lds_k0, buf, kv_row0); };
-  auto issue_v = [&](int buf, int kv_row0) { issue_tile(gV, true, lds_v0, buf, kv_row0); };
 
   // PARTIAL blocks: thread tid fetches 32 mask bytes of row tid/2 (a row of its own
   // wave), packs them to 32 bits and parks the word in LDS for the two lanes that own
   // the row.  Writer and readers are the same wave, so no workgroup barrier is needed.
-  // Done at the top of the step that needs it: no registers are held across steps for
-  // it, at the price of one exposed load latency per PARTIAL step.
+  // Done at the end of the iteration before the one that needs it.
   auto stage_mask_bits = [&](int it, const StepInfo& si) {
     const int half = it % SPB;
     const uint8_t* mp = p.partial_masks + size_t(si.pid) * (QB * KB) + size_t(tid >> 1) * KB +
@@ -344,180 +392,250 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     sBits[tid] = word;
   };
 
-  // Wave-uniform classification of this wave's 32x64 tile of a step:
-  // 0 = nothing to do, 1 = no mask needed, 2 = masked path.
-  auto classify = [&](const StepInfo& si) {
-    if (si.mode == kMasked) return 0;
-    const bool clip = si.row0 + STEP > p.seqlen;
-    if (si.mode == kCausal) {
-      if (si.row0 > q_wave_min + 31) return 0;                       // all in the future
-      if (si.row0 + STEP - 1 <= q_wave_min && !clip) return 1;       // all in the past
-      return 2;
-    }
-    return (si.mode == kFull && !clip) ? 1 : 2;
+  // Does this wave's 32x64 tile of the step need no mask at all?  (wave-uniform)
+  auto unmasked = [&](const StepInfo& si) {
+    if (si.row0 + STEP > p.seqlen) return false;
+    if (si.mode == kFull) return true;
+    return si.mode == kCausal && si.row0 + STEP - 1 <= q_wave_min;
   };
 
-  // S^T = K . Q^T for the 64 keys of one LDS tile: two 32-key accumulator tiles.
-  auto qk_tile = [&](const uint16_t* tK, f32x16_t (&st)[2]) {
-    const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const int row = 32 * t + c;
-        const int ch = (2 * s + g) ^ k_swizzle<D>(row);
-        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(tK + row * D + ch * 8);
-        st[t] = mfma_32x32x16<BF16>(a, qf[s], s == 0 ? zero : st[t]);
-      }
-    }
+  // LDS operand fetches.  K: rows 32t + c of the tile at k-step s.
+  auto k_frag = [&](const uint16_t* tK, int s, int t) {
+    const int row = 32 * t + c;
+    const int ch = (2 * s + g) ^ k_swizzle<D>(row);
+    return *reinterpret_cast<const u32x4_t*>(tK + row * D + ch * 8);
+  };
+  // V^T: operand j = (ts, dt) is rows 32 dt .. +31 of V^T (d) at keys 16 ts .. +15; k-slot e
+  // of lane group g in k-step ts = (t, s2) is key 32t + 16 s2 + 8(e/4) + 4g + e%4 -- the
+  // accumulator order of S^T.
+  const int i16 = c & 15;
+  const int j16 = c >> 4;
+  auto v_frag = [&](const uint16_t* tV, int j) {
+    const int ts = j / DT, dt = j % DT;
+    const int vrow = 16 * ts + 4 * g + (i16 >> 2);
+    const int unit = 2 * dt + j16;
+    const int u0 = unit ^ v_swizzle<D>(vrow);
+    const int u1 = unit ^ v_swizzle<D>(vrow + 8);
+    const s16x4_t lo = lds_read_tr16(tV + vrow * D + u0 * 16 + (i16 & 3) * 4);
+    const s16x4_t hi = lds_read_tr16(tV + (vrow + 8) * D + u1 * 16 + (i16 & 3) * 4);
+    const u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo);
+    const u32x2_t hi2 = __builtin_bit_cast(u32x2_t, hi);
+    const u32x4_t a = {lo2[0], lo2[1], hi2[0], hi2[1]};
+    return a;
   };
 
+  const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   f32x16_t ot[DT];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int dt = 0; dt < DT; ++dt) ot[dt] = zero16;
+  f32x16_t st[2][2];   // [set][32-key tile]: S^T of the current / next step, alternating
+  u32x4_t pb[2][2][2];  // [set][tile][16-key half]: P^T packed to 16 bits, B-operand order
 #pragma unroll
-    for (int r = 0; r < 16; ++r) ot[dt][r] = 0.f;
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      st[a][t] = zero16;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) pb[a][t][s2] = u32x4_t{0u, 0u, 0u, 0u};
+    }
   float m_run = -INFINITY;  // reference point of the exponentials, log2 domain (score * sl2)
   float l_run = 0.f;        // this lane's share of the running row sum
+  // When the reference point moves, the rescale of O waits until the top of the next
+  // iteration: the PV product that is in flight still belongs to the old reference.
+  float alpha_pending = 1.f;
+  uint64_t rescale_pending = 0;  // wave-uniform: lanes whose row outgrew the reference
 
-  // Mask (if needed) + online softmax of one step; leaves P (fp32) in st.
-  auto softmax_step = [&](f32x16_t (&st)[2], const StepInfo& si, bool masked_path) {
-    if (masked_path) {
-      // Register r of tile t holds key  row0 + 32t + 8(r/4) + 4g + r%4.
-      int limit = p.seqlen - 1;
-      if (si.mode == kCausal) limit = limit < q_row ? limit : q_row;
-      const int lim_l = limit - si.row0 - 4 * g;
-      uint32_t kw0 = 0xffffffffu, kw1 = 0xffffffffu;
-      if (si.mode == kPartial) {
-        const u32x2_t bw = *reinterpret_cast<const u32x2_t*>(sBits + (32 * w + c) * 2);
-        kw0 = bw[0];
-        kw1 = bw[1];
-      }
-      kw0 >>= 4 * g;
-      kw1 >>= 4 * g;
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const uint32_t kw = t == 0 ? kw0 : kw1;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int kl = 8 * (r >> 2) + (r & 3);
-          const bool keep = (32 * t + kl <= lim_l) && ((kw >> kl) & 1u);
-          st[t][r] = keep ? st[t][r] : -INFINITY;
-        }
-      }
+  // ---- one iteration of the pipeline ----------------------------------------------------
+  // SET = it % 2.  Reads K(it+1) from sK[SET^1] into st[SET^1], V(it-1) from sV[SET^1] with
+  // pb[SET^1]; softmax of st[SET] into pb[SET]; loads K(it+2) into sK[SET] and V(it) into
+  // sV[SET] (both last read one iteration ago).
+  constexpr int NQK = 2 * KS;    // MFMAs of S^T
+  constexpr int NPV = 4 * DT;    // MFMAs of O^T
+  constexpr int NS = NQK + NPV;  // slots
+  constexpr int NL = 2 * NCH;    // tile loads per thread
+  constexpr int LSP = (NS / 2) / NL > 0 ? (NS / 2) / NL : 1;  // slots between tile loads
+  constexpr int PF = NS < 4 ? NS : 4;                        // operand fetch distance
+  static_assert(NL * LSP <= NS, "tile loads must fit in the slots");
+  constexpr float kSlack = 6.f;
+
+  // Mask of a step whose 32x64 tile is not entirely allowed, applied to S^T before the
+  // iteration that does its softmax: disallowed scores become -inf.  Register r of tile t
+  // holds key  row0 + 32t + 8(r/4) + 4g + r%4.
+  auto apply_mask = [&](auto set_c, const StepInfo& si) {
+    constexpr int SET = decltype(set_c)::value;
+    int limit = p.seqlen - 1;
+    if (si.mode == kCausal) limit = limit < q_row ? limit : q_row;
+    if (si.mode == kMasked) limit = -1;
+    const int lim_l = limit - si.row0 - 4 * g;
+    uint32_t kw[2] = {0xffffffffu, 0xffffffffu};
+    if (si.mode == kPartial) {
+      const u32x2_t bw = *reinterpret_cast<const u32x2_t*>(sBits + (32 * w + c) * 2);
+      kw[0] = bw[0];
+      kw[1] = bw[1];
     }
-    // The row lives in lanes c and c+32.
-    float mx = st[0][0];
+    kw[0] >>= 4 * g;
+    kw[1] >>= 4 * g;
+    static_for<32>([&](auto ec) {
+      constexpr int e = decltype(ec)::value;
+      constexpr int t = e / 16, r = e % 16;
+      constexpr int kl = 8 * (r >> 2) + (r & 3);
+      const bool keep = (32 * t + kl <= lim_l) && ((kw[t] >> kl) & 1u);
+      st[SET][t][r] = keep ? st[SET][t][r] : -INFINITY;
+    });
+  };
+
+  auto body = [&](auto set_c, int k_row0, int v_row0) {
+    constexpr int SET = decltype(set_c)::value;
+    constexpr int NV = 4 + 1 + 16;  // vector chunks: max, reference, 16 exp pairs
+    const uint16_t* tK = sK + (SET ^ 1) * TILE;
+    const uint16_t* tV = sV + (SET ^ 1) * TILE;
+    auto operand = [&](int n) { return n < NPV ? v_frag(tV, n) : k_frag(tK, (n - NPV) / 2, (n - NPV) % 2); };
+
+    u32x4_t opq[PF];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int n = 0; n < PF; ++n) opq[n] = operand(n);
+
+    float mxa = -INFINITY, mxb = -INFINITY, m_ref = 0.f, rs0 = 0.f, rs1 = 0.f;
+    auto vector_chunk = [&](auto uc) {
+      constexpr int u = decltype(uc)::value;
+      if constexpr (u < 0) {
+      } else if constexpr (u < 4) {
+        static_for<8>([&](auto ec) {
+          constexpr int e = 8 * u + decltype(ec)::value;
+          if constexpr ((u & 1) != 0) {
+            mxb = fmaxf(mxb, st[SET][e / 16][e % 16]);
+          } else {
+            mxa = fmaxf(mxa, st[SET][e / 16][e % 16]);
+          }
+        });
+        pin(mxa, mxb);
+      } else if constexpr (u == 4) {
+        // The reference point m_run of the exponentials only has to stay within 2^kSlack of
+        // the true running max (P then stays below 2^kSlack, exact in fp32 and well inside
+        // the 16-bit types' range), so it is moved -- and O, l rescaled -- only when some
+        // row of the wave outgrows it by more than that.  The decision is wave-uniform; the
+        // result is the same sum with a different common factor.  (Written without
+        // branches: an unmoved reference gives a factor of exactly 1, or of 0 for a row that
+        // has not seen a key yet and whose sums are still 0.)
+        const float mx = pair_max(fmaxf(mxa, mxb));  // the row lives in lanes c and c+32
+        const float m_cand = mx * p.sl2;
+        const uint64_t movers = __builtin_amdgcn_ballot_w64(m_cand > m_run + kSlack);
+        const bool move = movers != 0;
+        const float m_new = move ? fmaxf(m_run, m_cand) : m_run;
+        m_ref = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+        l_run *= alpha;
+        m_run = m_new;
+        alpha_pending = move ? alpha : alpha_pending;
+        rescale_pending |= movers;
+        pin(l_run, alpha_pending);
+      } else {
+        constexpr int i = u - 5;
+        constexpr int t = i / 8, r = 2 * (i % 8);
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[SET][t][r], p.sl2, -m_ref));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[SET][t][r + 1], p.sl2, -m_ref));
+        rs0 += p0;
+        rs1 += p1;
+        uint32_t packed = pack2<BF16>(p0, p1);
+        pin(packed);
+        pb[SET][t][r >> 3][(r & 7) >> 1] = packed;
+        pin(rs0, rs1);
+        if constexpr (i == 15) l_run += rs0 + rs1;
+      }
+    };
+
+    static_for<NS>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      if constexpr (j < NPV) {
+        constexpr int ts = j / DT, dt = j % DT;
+        ot[dt] = mfma_32x32x16<BF16>(opq[j % PF], pb[SET ^ 1][ts >> 1][ts & 1], ot[dt]);
+      } else {
+        constexpr int s = (j - NPV) / 2, t = (j - NPV) % 2;
+        st[SET ^ 1][t] = mfma_32x32x16<BF16>(opq[j % PF], qf[s], s == 0 ? zero16 : st[SET ^ 1][t]);
+      }
+      if constexpr (j + PF < NS) opq[j % PF] = operand(j + PF);
+      if constexpr (j % LSP == 0 && j / LSP < NL) issue_load(j / LSP, SET, k_row0, v_row0);
+      constexpr int u_lo = j * NV / NS, u_hi = (j + 1) * NV / NS;
+      static_for<u_hi - u_lo>([&](auto dc) { vector_chunk(IntC<u_lo + decltype(dc)::value>{}); });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+
+  // ---- the walk -------------------------------------------------------------------------
+  StepInfo cur = {0, kMasked, -1}, nxt = cur, nn = cur;
+  if (nsteps > 0) {
+    load_chunk(0);
+    cur = step_info(0);
+    nxt = step_info(1);
+    nn = step_info(2);
+    // Prologue: K(0) and K(1); the V buffer that iteration 0 multiplies with its all-zero P
+    // is cleared (0 * stale LDS contents could be NaN).
+    {
+      u32x4_t* z = reinterpret_cast<u32x4_t*>(sV + TILE);
+      for (int i = tid; i < TILE * 2 / 16; i += NT) z[i] = u32x4_t{0u, 0u, 0u, 0u};
+    }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[t][r]);
-    mx = pair_max(mx);
-    // The reference point m_run of the exponentials only has to stay within 2^kSlack of
-    // the true running max (P then stays below 2^kSlack, exact in fp32 and well inside
-    // the 16-bit types' range), so it is moved -- and O, l rescaled -- only when some
-    // row of the wave outgrows it by more than that.  The decision is wave-uniform; the
-    // result is the same sum with a different common factor.
-    constexpr float kSlack = 6.f;
-    const float m_cand = mx * p.sl2;
-    if (__builtin_amdgcn_ballot_w64(m_cand > m_run + kSlack) != 0) {
-      const float m_new = fmaxf(m_run, m_cand);
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);  // m_run = -inf -> 0
-      m_run = m_new;
-      l_run *= alpha;
+    for (int i = 0; i < NCH; ++i) {
+      issue_load(NCH + i, 0, cur.row0, 0);
+      issue_load(NCH + i, 1, nxt.row0, 0);
+    }
+    if (cur.mode == kPartial) stage_mask_bits(0, cur);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        st[0][t] = mfma_32x32x16<BF16>(k_frag(sK, s, t), qf[s], s == 0 ? zero16 : st[0][t]);
+  }
+
+  auto iteration = [&](auto set_c, int it) {
+    constexpr int SET = decltype(set_c)::value;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's tile loads have landed
+    __syncthreads();
+    if (rescale_pending != 0) {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) ot[dt][r] *= alpha;
+        for (int r = 0; r < 16; ++r) ot[dt][r] *= alpha_pending;
+      rescale_pending = 0;
     }
-    const float m_ref = m_run == -INFINITY ? 0.f : m_run;
-    float rs = 0.f;
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(st[t][r], p.sl2, -m_ref));
-        st[t][r] = pv;
-        rs += pv;
-      }
-    l_run += rs;
+    if (!unmasked(cur)) apply_mask(IntC<SET>{}, cur);
+    body(IntC<SET>{}, nn.row0, cur.row0);
+    if (it + 1 < nsteps && nxt.mode == kPartial) stage_mask_bits(it + 1, nxt);
+    const StepInfo n3 = step_info(it + 3);
+    cur = nxt;
+    nxt = nn;
+    nn = n3;
   };
-
-  // O^T += V^T . P^T.  k-slot e of lane group g in k-step (t, s2) is key
-  // 32t + 16 s2 + 8(e/4) + 4g + e%4 -- the accumulator order of S^T.
-  auto pv_tile = [&](const uint16_t* tV, const f32x16_t (&st)[2]) {
-    const int i16 = c & 15;
-    const int j16 = c >> 4;
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        u32x4_t pb;
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          pb[e] = pack2<BF16>(st[t][8 * s2 + 2 * e], st[t][8 * s2 + 2 * e + 1]);
-        const int vrow = 32 * t + 16 * s2 + 4 * g + (i16 >> 2);
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const int unit = 2 * dt + j16;
-          const int u0 = unit ^ v_swizzle<D>(vrow);
-          const int u1 = unit ^ v_swizzle<D>(vrow + 8);
-          const s16x4_t lo = lds_read_tr16(tV + vrow * D + u0 * 16 + (i16 & 3) * 4);
-          const s16x4_t hi = lds_read_tr16(tV + (vrow + 8) * D + u1 * 16 + (i16 & 3) * 4);
-          const u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo);
-          const u32x2_t hi2 = __builtin_bit_cast(u32x2_t, hi);
-          const u32x4_t a = {lo2[0], lo2[1], hi2[0], hi2[1]};
-          ot[dt] = mfma_32x32x16<BF16>(a, pb, ot[dt]);
-        }
-      }
-    }
-  };
-
-  // ---- software pipeline ----------------------------------------------------------
-  // Top of iteration `it` (before the barrier): in flight are K(it+1) -> sK[(it+1)&1] and
-  // V(it) -> sV[it&1]; st_cur holds S^T of step it.  After the barrier every wave has
-  // finished reading sK[it&1] (S^T of step it) and sV[(it-1)&1] (PV of step it-1), so
-  // those two buffers are refilled with K(it+2) and V(it+1).
-  // Step descriptors: raw metadata words are loaded three steps ahead and interpreted
-  // one iteration later, two steps ahead of their first use (the K tile load).
-  StepInfo cur = interpret(0, fetch_raw(0));
-  StepInfo nxt = interpret(1, fetch_raw(1));
-  StepInfo nn = interpret(2, fetch_raw(2));
-  RawStep raw3 = fetch_raw(3);
-  int cls_cur = classify(cur), cls_nxt = nsteps > 1 ? classify(nxt) : 0;
-  f32x16_t st_cur[2], st_nxt[2];
-  if (nsteps > 0) {
-    issue_k(0, cur.row0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __syncthreads();
-    if (nsteps > 1) issue_k(1, nxt.row0);
-    issue_v(0, cur.row0);
-    if (cls_cur != 0) qk_tile(sK, st_cur);
+  for (int it = 0; it < nsteps; it += 2) {
+    iteration(IntC<0>{}, it);
+    if (it + 1 < nsteps) iteration(IntC<1>{}, it + 1);
   }
 
-  for (int it = 0; it < nsteps; ++it) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's tile loads have landed
+  // Drain: O^T += V^T . P^T of the last step.
+  if (nsteps > 0) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    if (it + 2 < nsteps) issue_k(it & 1, nn.row0);
-    if (it + 1 < nsteps) issue_v((it + 1) & 1, nxt.row0);
-    const StepInfo n3 = interpret(it + 3, raw3);
-    raw3 = fetch_raw(it + 4);
-    if (cur.mode == kPartial) stage_mask_bits(it, cur);
-
-    if (cls_nxt != 0) qk_tile(sK + ((it + 1) & 1) * TILE, st_nxt);
-    if (cls_cur != 0) {
-      softmax_step(st_cur, cur, cls_cur == 2);
-      pv_tile(sV + (it & 1) * TILE, st_cur);
-    }
-
+    if (rescale_pending != 0) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) st_cur[t] = st_nxt[t];
-    cur = nxt;
-    cls_cur = cls_nxt;
-    nxt = nn;
-    cls_nxt = (it + 2 < nsteps) ? classify(nn) : 0;
-    nn = n3;
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ot[dt][r] *= alpha_pending;
+    }
+    auto drain = [&](auto set_c) {
+      constexpr int SET = decltype(set_c)::value;
+#pragma unroll
+      for (int j = 0; j < NPV; ++j) {
+        const int ts = j / DT, dt = j % DT;
+        ot[dt] = mfma_32x32x16<BF16>(v_frag(sV + SET * TILE, j), pb[SET][ts >> 1][ts & 1], ot[dt]);
+      }
+    };
+    if ((nsteps - 1) & 1) {
+      drain(IntC<1>{});
+    } else {
+      drain(IntC<0>{});
+    }
   }
 
   // Epilogue: O = O^T / l, zeros for rows without any allowed key or beyond seqlen.
