@@ -24,7 +24,7 @@
 // MFMAs of S^T(i+1) and the D/8 MFMAs of O^T += V^T.P^T(i-1) while its vector
 // instructions do the online softmax of step i.  None of the three depends on another
 // inside the iteration, and the source spells the interleaving out: the iteration is a
-// sequence of slots, each with one MFMA, the LDS fetch of the operand four slots ahead, a
+// sequence of slots, each with one MFMA, the LDS fetch of the operand three slots ahead, a
 // share of the softmax and -- in the early slots -- one tile load, with a scheduling fence
 // after every slot.  (A wave that issues MFMAs back to back leaves other waves of its
 // SIMD almost no vector issue slots; vector instructions placed between the MFMAs of the
@@ -298,27 +298,32 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
 
   const size_t meta_row = size_t(bh) * p.Tq + qb;
   const size_t meta_off = meta_row * p.max_blocks;
+
+  // Block metadata lives in registers: lane i of every wave holds the (validated) words of
+  // block 64 * chunk + i of this query block's list -- first key row, effective mode,
+  // partial-mask index -- and a step's words are picked out with v_readlane: no memory
+  // instruction per step.  A new chunk is fetched when the walk reaches it (every 64
+  // blocks).  The loads of a chunk do not depend on the block count, so the first chunk,
+  // the count and Q are all in flight together at the start of the kernel.
+  const bool has_partial = p.partial_idx != nullptr && p.partial_masks != nullptr;
+  int32_t mv_row0 = 0, mv_mode = kMasked, mv_pid = -1;
+  auto load_chunk = [&](int chunk) {
+    const int j = chunk * 64 + lane;
+    const size_t o = meta_off + size_t(j < p.max_blocks ? j : 0);
+    const int32_t kvb_raw = p.kv_indices[o];
+    const int32_t ty = p.types[o];
+    const int32_t pid = has_partial ? p.partial_idx[o] : -1;
+    const int32_t kvb = kvb_raw < 0 ? 0 : (kvb_raw >= p.Tk ? p.Tk - 1 : kvb_raw);
+    int32_t mode = (ty == kCausal || ty == kFull || ty == kPartial) ? ty : int32_t(kMasked);
+    if (ty == kPartial && pid < 0) mode = kMasked;
+    mv_row0 = kvb * KB;
+    mv_mode = mode;
+    mv_pid = pid;
+  };
+  load_chunk(0);
   int nb = load_uniform(p.kv_num_blocks + meta_row);
   nb = nb < 0 ? 0 : (nb > p.max_blocks ? p.max_blocks : nb);
   const int nsteps = nb * SPB;
-
-  // Block metadata lives in registers: lane i of every wave holds the three words of
-  // block 64 * chunk + i of this query block's list, and a step's words are picked out
-  // with v_readlane -- no memory instruction per step.  A new chunk is fetched when the
-  // walk reaches it (every 64 blocks).
-  const bool has_partial = p.partial_idx != nullptr && p.partial_masks != nullptr;
-  int32_t mv_kvb = 0, mv_ty = kMasked, mv_pid = -1;
-  auto load_chunk = [&](int chunk) {
-    const int j = chunk * 64 + lane;
-    const bool ok = j < nb;
-    const size_t o = meta_off + size_t(ok ? j : 0);
-    const int32_t kvb = p.kv_indices[o];
-    const int32_t ty = p.types[o];
-    const int32_t pid = has_partial ? p.partial_idx[o] : -1;
-    mv_kvb = ok ? kvb : 0;
-    mv_ty = ok ? ty : int32_t(kMasked);
-    mv_pid = ok ? pid : -1;
-  };
   // Step `it` (clamped to the last step of the walk; steps past the end are only ever
   // used as the address of a tile load whose data nobody reads).
   auto step_info = [&](int it) {
@@ -326,15 +331,10 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     const int j = itc / SPB;
     if (itc == it && itc % SPB == 0 && (j & 63) == 0 && j > 0) load_chunk(j >> 6);
     const int ln = j & 63;
-    const int kvb_raw = __builtin_amdgcn_readlane(mv_kvb, ln);
-    const int ty = __builtin_amdgcn_readlane(mv_ty, ln);
-    const int pid = __builtin_amdgcn_readlane(mv_pid, ln);
     StepInfo si;
-    const int kvb = kvb_raw < 0 ? 0 : (kvb_raw >= p.Tk ? p.Tk - 1 : kvb_raw);
-    si.mode = (ty == kCausal || ty == kFull || ty == kPartial) ? ty : kMasked;
-    si.pid = pid;
-    if (ty == kPartial && pid < 0) si.mode = kMasked;
-    si.row0 = kvb * KB + (itc % SPB) * STEP;
+    si.row0 = __builtin_amdgcn_readlane(mv_row0, ln) + (itc % SPB) * STEP;
+    si.mode = __builtin_amdgcn_readlane(mv_mode, ln);
+    si.pid = __builtin_amdgcn_readlane(mv_pid, ln);
     return si;
   };
 
@@ -454,7 +454,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   constexpr int NS = NQK + NPV;  // slots
   constexpr int NL = 2 * NCH;    // tile loads per thread
   constexpr int LSP = (NS / 2) / NL > 0 ? (NS / 2) / NL : 1;  // slots between tile loads
-  constexpr int PF = NS < 4 ? NS : 4;                        // operand fetch distance
+  constexpr int PF = 3;                                      // operand fetch distance in slots
   static_assert(NL * LSP <= NS, "tile loads must fit in the slots");
   constexpr float kSlack = 6.f;
 
@@ -564,7 +564,6 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   // ---- the walk -------------------------------------------------------------------------
   StepInfo cur = {0, kMasked, -1}, nxt = cur, nn = cur;
   if (nsteps > 0) {
-    load_chunk(0);
     cur = step_info(0);
     nxt = step_info(1);
     nn = step_info(2);
