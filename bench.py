@@ -8,6 +8,7 @@ Prints ONE JSON line.  `value` is effective TFLOP/s: 4*QB*KB*D flops per listed
 not counted, EMPTY blocks count nothing -- divided by the wall time per step.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+    python bench.py --sweep-bands     # runtime against the number of listed blocks (fixed shape)
 """
 import argparse
 import json
@@ -62,6 +63,72 @@ def cpu_baseline(w, budget_s: float):
     }
 
 
+def band_sweep(dev, steps, warmup):
+    """Kernel time against the number of listed blocks at the fixed shape of c2_interleaved
+    (B=2, H=32, S=4096, D=128, bf16, 128/128): banded masks, query block i lists the FULL
+    blocks max(0, i-w+1) .. i, for band widths w = 1, 2, 4, ... Tk.  Least-squares fit
+    t = a + b * N_ne; returns the fit and the points."""
+    import torch
+
+    import omni_attn_capi
+
+    B, H, S, D, QB, KB = 2, 32, 4096, 128, 128, 128
+    Tq, Tk = S // QB, S // KB
+    g = torch.Generator(device="cpu").manual_seed(0)
+    q, k, v = (torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(dev) for _ in range(3))
+    o = torch.empty_like(q)
+    stream = torch.cuda.current_stream(dev)
+    points = []
+    w = 1
+    while w <= Tk:
+        nb = torch.zeros(Tq, dtype=torch.int32)
+        idx = torch.zeros(Tq, Tk, dtype=torch.int32)
+        for i in range(Tq):
+            lo = max(0, i - w + 1)
+            nb[i] = i - lo + 1
+            idx[i, : i - lo + 1] = torch.arange(lo, i + 1, dtype=torch.int32)
+        tys = torch.full((Tq, Tk), 2, dtype=torch.int32)
+        nb_d = nb.expand(B, H, Tq).contiguous().to(dev)
+        idx_d = idx.expand(B, H, Tq, Tk).contiguous().to(dev)
+        tys_d = tys.expand(B, H, Tq, Tk).contiguous().to(dev)
+
+        def step():
+            omni_attn_capi.fwd(q, k, v, o, None, nb_d, idx_d, tys_d, QB, KB, S, None, None,
+                               stream=stream.cuda_stream)
+
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        for i in range(steps):
+            starts[i].record(stream)
+            step()
+            ends[i].record(stream)
+        torch.cuda.synchronize()
+        ms = statistics.median(a.elapsed_time(b) for a, b in zip(starts, ends))
+        n_ne = int(nb.sum()) * B * H
+        points.append({"band_blocks": w, "nonempty_blocks": n_ne, "kernel_ms_median": ms,
+                       "tflops": 4.0 * QB * KB * D * n_ne / (ms * 1e-3) / 1e12})
+        w *= 2
+    xs = [p["nonempty_blocks"] for p in points]
+    ys = [p["kernel_ms_median"] for p in points]
+    n = len(xs)
+    mx, my = sum(xs) / n, sum(ys) / n
+    sxx = sum((x - mx) ** 2 for x in xs)
+    sxy = sum((x - mx) * (y - my) for x, y in zip(xs, ys))
+    b = sxy / sxx
+    a = my - b * mx
+    ss_res = sum((y - (a + b * x)) ** 2 for x, y in zip(xs, ys))
+    ss_tot = sum((y - my) ** 2 for y in ys)
+    return {
+        "sweep": "banded FULL masks, B=2 H=32 S=4096 D=128 bf16, Q_BLOCK=KV_BLOCK=128",
+        "fit": {"ms_fixed": a, "ns_per_block": b * 1e6, "r2": 1.0 - ss_res / ss_tot,
+                "max_rel_residual": max(abs(y - (a + b * x)) / y for x, y in zip(xs, ys))},
+        "points": points,
+    }
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -74,6 +141,8 @@ def main(argv=None):
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, so that a counter run of this "
                          "command shows what FETCH_SIZE / WRITE_SIZE read for a known traffic")
+    ap.add_argument("--sweep-bands", action="store_true",
+                    help="instead of the workload: kernel time against the number of listed blocks")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py measures one GPU: (batch, head) slabs are independent, so more GPUs would "
@@ -91,6 +160,9 @@ def main(argv=None):
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     omni_attn_capi.load_library()  # fail loudly when the HIP library is missing
+    if args.sweep_bands:
+        print(json.dumps(band_sweep(dev, min(args.steps, 30), min(args.warmup, 5))))
+        return 0
 
     w = make_workload(args.workload, seed=args.seed)
     m = w.block_mask
@@ -149,7 +221,7 @@ def main(argv=None):
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": w.info["dtype"],
+        "dtype": {"bfloat16": "bf16", "float16": "f16"}.get(w.info["dtype"], w.info["dtype"]),
         "data": "synthetic",
         "config": {
             "workload": f"{w.name}: B={B} H={H} S={S} D={D} {w.info['dtype']}, Q_BLOCK={m.Q_BLOCK_SIZE} "

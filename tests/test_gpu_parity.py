@@ -179,3 +179,29 @@ def test_runs_are_bitwise_reproducible(gpu_device):
     a = run_workload(w, gpu_device)
     b = run_workload(w, gpu_device)
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+@pytest.mark.parametrize("QB,KB,D", [(64, 64, 32), (128, 64, 64)])
+def test_more_than_64_listed_blocks_per_query_block(QB, KB, D, gpu_device):
+    """Lists longer than 64 and 128 blocks (the kernel keeps 64 blocks of metadata in
+    registers and fetches the next 64 when the walk gets there), random slot kinds."""
+    gen = torch.Generator().manual_seed(77 + D)
+    B, H, S = 1, 2, 64 * 134
+    dtype = torch.float16
+    q, k, v = (torch.randn(B, H, S, D, generator=gen).to(dtype) for _ in range(3))
+    nb, idx, tys, pidx, pm = random_block_metadata(gen, B, H, S // QB, S // KB, QB, KB, p_empty=0.05,
+                                                   shuffle=True)
+    assert int(nb.max()) > 128
+    o, lse = run_kernel(q, k, v, nb, idx, tys, QB, KB, S - 10, pidx, pm, device=gpu_device)
+    wo, wl = attention_block_walk(q, k, v, nb, idx, tys, QB, KB, S - 10, pidx, pm)
+    compare_with_oracle(o, lse, wo, wl, dtype, "block walk, long lists")
+
+
+def test_runtime_is_linear_in_listed_blocks(gpu_device):
+    """Kernel time against the number of listed blocks at a fixed shape (banded masks of
+    width 1, 2, 4 ... 32 blocks): a straight line, t = a + b * N_ne."""
+    import bench
+
+    r = bench.band_sweep(torch.device(gpu_device), steps=12, warmup=3)
+    assert r["fit"]["r2"] > 0.99, r
+    assert r["fit"]["ns_per_block"] > 0
