@@ -287,15 +287,6 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   const int q_row = qb * QB + 32 * w + c;  // this lane's query row inside the slab
   const int q_wave_min = qb * QB + 32 * w;
 
-  // Q as the B operand of S^T = K.Q^T: lane holds Q[q_row][16s + 8g .. +7].
-  u32x4_t qf[KS];
-  {
-    const int qr = q_row < p.S ? q_row : p.S - 1;
-    const uint16_t* qp = p.q + slab + size_t(qr) * D + 8 * g;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const u32x4_t*>(qp + 16 * s);
-  }
-
   const size_t meta_row = size_t(bh) * p.Tq + qb;
   const size_t meta_off = meta_row * p.max_blocks;
 
@@ -324,6 +315,15 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   int nb = load_uniform(p.kv_num_blocks + meta_row);
   nb = nb < 0 ? 0 : (nb > p.max_blocks ? p.max_blocks : nb);
   const int nsteps = nb * SPB;
+
+  // Q as the B operand of S^T = K.Q^T: lane holds Q[q_row][16s + 8g .. +7].
+  u32x4_t qf[KS];
+  {
+    const int qr = q_row < p.S ? q_row : p.S - 1;
+    const uint16_t* qp = p.q + slab + size_t(qr) * D + 8 * g;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const u32x4_t*>(qp + 16 * s);
+  }
   // Step `it` (clamped to the last step of the walk; steps past the end are only ever
   // used as the address of a tile load whose data nobody reads).
   auto step_info = [&](int it) {
@@ -638,11 +638,16 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   }
 
   // Epilogue: O = O^T / l, zeros for rows without any allowed key or beyond seqlen.
+  // A lane holds 4 consecutive d of its row per accumulator group; stored directly, one
+  // store instruction would touch 32 rows with 16 bytes each.  So the wave transposes its
+  // 32 x D output through LDS -- its own 32 rows of the K buffers, which nobody reads after
+  // the barrier of the drain, 16-byte chunks swizzled like a K tile -- and stores whole
+  // rows: 64 lanes x 16 bytes = 64 / CPR complete rows per instruction.
   const float l_tot = pair_sum(l_run);
   const bool live = (q_row < p.seqlen) && (l_tot > 0.f);
   const float inv = live ? 1.f / l_tot : 0.f;
-  if (q_row < p.S) {
-    uint16_t* op = p.o + slab + size_t(q_row) * D + 4 * g;
+  {
+    uint16_t* stage = sK + size_t(w) * 32 * D;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
@@ -650,13 +655,24 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
         u32x2_t ov;
         ov[0] = pack2<BF16>(ot[dt][4 * r4 + 0] * inv, ot[dt][4 * r4 + 1] * inv);
         ov[1] = pack2<BF16>(ot[dt][4 * r4 + 2] * inv, ot[dt][4 * r4 + 3] * inv);
-        *reinterpret_cast<u32x2_t*>(op + 32 * dt + 8 * r4) = ov;
+        const int ch = (4 * dt + r4) ^ k_swizzle<D>(c);
+        *reinterpret_cast<u32x2_t*>(stage + c * D + ch * 8 + 4 * g) = ov;
       }
     }
-    if (p.lse != nullptr && g == 0) {
-      const float lse = live ? (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : -INFINITY;
-      p.lse[size_t(bh) * p.S + q_row] = lse;
+    constexpr int ROWS_PER_STORE = 64 / CPR;
+    const int srow = lane / CPR, pch = lane % CPR;
+#pragma unroll
+    for (int i = 0; i < 32 / ROWS_PER_STORE; ++i) {
+      const int row = i * ROWS_PER_STORE + srow;  // row of the wave
+      const u32x4_t val = *reinterpret_cast<const u32x4_t*>(stage + row * D + pch * 8);
+      const int grow = q_wave_min + row;
+      if (grow < p.S)
+        *reinterpret_cast<u32x4_t*>(p.o + slab + size_t(grow) * D + (pch ^ k_swizzle<D>(row)) * 8) = val;
     }
+  }
+  if (q_row < p.S && p.lse != nullptr && g == 0) {
+    const float lse = live ? (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : -INFINITY;
+    p.lse[size_t(bh) * p.S + q_row] = lse;
   }
 }
 
