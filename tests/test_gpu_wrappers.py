@@ -2,6 +2,7 @@
 import pytest
 import torch
 
+import omni_attn_torch as oat
 from baseline_configs import make_workload
 from helpers import compare_with_oracle
 from omni_attn_torch import (create_causal_omni_block_mask, create_omni_block_mask_from_modality_positions,
@@ -9,6 +10,8 @@ from omni_attn_torch import (create_causal_omni_block_mask, create_omni_block_ma
                              omni_attention_preftech, omni_attention_shared_kv,
                              omni_attention_shared_kv_swizzle, omni_attention_simple)
 from oracle.dense_oracle import attention_dense_fp32
+
+
 
 pytestmark = pytest.mark.gpu
 
@@ -85,3 +88,32 @@ def test_module_errors_on_gpu_tensors(gpu_device):
     # and a good call still works afterwards
     omni_attn.omni_attn_simple_kernel(q, q, q, q.clone(), nb, idx, torch.full_like(idx, 2), 128, 128, 256, e_i, e_b, False)
     torch.cuda.synchronize()
+
+
+def test_mask_builders_run_on_the_gpu_and_agree_with_the_cpu(gpu_device):
+    """The Transfusion-rule builder is plain tensor algebra: built on the GPU from
+    modality positions it gives the metadata the CPU build gives, and the wrapper accepts
+    it as is (no host round trip of the mask)."""
+    import time
+
+    S, H = 16384, 4
+    mp = torch.tensor([[[1, 700, 1024], [1, 5000, 900], [1, 9000, 1500], [0, 0, 0]],
+                       [[1, 128, 1024], [1, 4096, 2048], [1, 12000, 1111], [1, 15000, 1384]]])
+    cpu = oat.create_omni_block_mask_from_modality_positions(mp, 2, H, S, S, 128, 128, device="cpu")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    gpu = oat.create_omni_block_mask_from_modality_positions(mp, 2, H, S, S, 128, 128, device=gpu_device)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    for name in ("kv_num_blocks", "kv_indices", "block_mask_types", "partial_block_mask_indices",
+                 "partial_block_masks"):
+        a, b = getattr(cpu, name), getattr(gpu, name)
+        assert b.is_cuda and torch.equal(a, b.cpu()), name
+    assert dt < 5.0, f"GPU mask build took {dt:.2f} s"
+    g = torch.Generator().manual_seed(3)
+    q, k, v = (torch.randn(2, H, 2048, 64, generator=g).to(torch.float16).to(gpu_device) for _ in range(3))
+    small = oat.create_omni_block_mask_from_modality_positions(mp[:, :1] // 8 * 2, 2, H, 2048, 2048, 64, 64,
+                                                               device=gpu_device)
+    o = oat.omni_attention_shared_kv(q, k, v, small)
+    ref = torch.nan_to_num(oat.naive_attention(q.float(), k.float(), v.float(), small), nan=0.0)
+    assert (o.float() - ref).abs().max().item() <= 2e-3
