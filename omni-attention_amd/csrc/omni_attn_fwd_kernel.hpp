@@ -449,13 +449,10 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   // SET = it % 2.  Reads K(it+1) from sK[SET^1] into st[SET^1], V(it-1) from sV[SET^1] with
   // pb[SET^1]; softmax of st[SET] into pb[SET]; loads K(it+2) into sK[SET] and V(it) into
   // sV[SET] (both last read one iteration ago).
-  constexpr int NQK = 2 * KS;    // MFMAs of S^T
-  constexpr int NPV = 4 * DT;    // MFMAs of O^T
-  constexpr int NS = NQK + NPV;  // slots
-  constexpr int NL = 2 * NCH;    // tile loads per thread
-  constexpr int LSP = (NS / 2) / NL > 0 ? (NS / 2) / NL : 1;  // slots between tile loads
-  constexpr int PF = 3;                                      // operand fetch distance in slots
-  static_assert(NL * LSP <= NS, "tile loads must fit in the slots");
+  constexpr int NQK = 2 * KS;     // MFMAs of S^T
+  constexpr int NPV_ALL = 4 * DT; // MFMAs of O^T
+  constexpr int NL = 2 * NCH;     // tile loads per thread
+  constexpr int PF_ALL = 3;       // operand fetch distance in slots
   constexpr float kSlack = 6.f;
 
   // Mask of a step whose 32x64 tile is not entirely allowed, applied to S^T before the
@@ -484,8 +481,14 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     });
   };
 
-  auto body = [&](auto set_c, int k_row0, int v_row0) {
+  auto body = [&](auto set_c, auto first_c, int k_row0, int v_row0) {
     constexpr int SET = decltype(set_c)::value;
+    // The first iteration of a walk has no previous step: no PV slots.
+    constexpr int NPV = decltype(first_c)::value != 0 ? 0 : NPV_ALL;
+    constexpr int NS = NQK + NPV;  // slots
+    constexpr int LSP = (NS / 2) / NL > 0 ? (NS / 2) / NL : 1;  // slots between tile loads
+    static_assert(NL * LSP <= NS, "tile loads must fit in the slots");
+    constexpr int PF = PF_ALL < NS ? PF_ALL : NS;
     constexpr int NV = 4 + 1 + 16;  // vector chunks: max, reference, 16 exp pairs
     const uint16_t* tK = sK + (SET ^ 1) * TILE;
     const uint16_t* tV = sV + (SET ^ 1) * TILE;
@@ -567,12 +570,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     cur = step_info(0);
     nxt = step_info(1);
     nn = step_info(2);
-    // Prologue: K(0) and K(1); the V buffer that iteration 0 multiplies with its all-zero P
-    // is cleared (0 * stale LDS contents could be NaN).
-    {
-      u32x4_t* z = reinterpret_cast<u32x4_t*>(sV + TILE);
-      for (int i = tid; i < TILE * 2 / 16; i += NT) z[i] = u32x4_t{0u, 0u, 0u, 0u};
-    }
+    // Prologue: K(0) and K(1).
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       issue_load(NCH + i, 0, cur.row0, 0);
@@ -588,7 +586,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
         st[0][t] = mfma_32x32x16<BF16>(k_frag(sK, s, t), qf[s], s == 0 ? zero16 : st[0][t]);
   }
 
-  auto iteration = [&](auto set_c, int it) {
+  auto iteration = [&](auto set_c, auto first_c, int it) {
     constexpr int SET = decltype(set_c)::value;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's tile loads have landed
     __syncthreads();
@@ -600,16 +598,20 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
       rescale_pending = 0;
     }
     if (!unmasked(cur)) apply_mask(IntC<SET>{}, cur);
-    body(IntC<SET>{}, nn.row0, cur.row0);
+    body(IntC<SET>{}, first_c, nn.row0, cur.row0);
     if (it + 1 < nsteps && nxt.mode == kPartial) stage_mask_bits(it + 1, nxt);
     const StepInfo n3 = step_info(it + 3);
     cur = nxt;
     nxt = nn;
     nn = n3;
   };
-  for (int it = 0; it < nsteps; it += 2) {
-    iteration(IntC<0>{}, it);
-    if (it + 1 < nsteps) iteration(IntC<1>{}, it + 1);
+  if (nsteps > 0) {
+    iteration(IntC<0>{}, IntC<1>{}, 0);
+    if (1 < nsteps) iteration(IntC<1>{}, IntC<0>{}, 1);
+  }
+  for (int it = 2; it < nsteps; it += 2) {
+    iteration(IntC<0>{}, IntC<0>{}, it);
+    if (it + 1 < nsteps) iteration(IntC<1>{}, IntC<0>{}, it + 1);
   }
 
   // Drain: O^T += V^T . P^T of the last step.
@@ -625,7 +627,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     auto drain = [&](auto set_c) {
       constexpr int SET = decltype(set_c)::value;
 #pragma unroll
-      for (int j = 0; j < NPV; ++j) {
+      for (int j = 0; j < NPV_ALL; ++j) {
         const int ts = j / DT, dt = j % DT;
         ot[dt] = mfma_32x32x16<BF16>(v_frag(sV + SET * TILE, j), pb[SET][ts >> 1][ts & 1], ot[dt]);
       }
