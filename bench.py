@@ -132,8 +132,10 @@ def band_sweep(dev, steps, warmup):
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=100,
+                    help="untimed launches first; the shader clock takes some tens of milliseconds of "
+                         "load to settle, a short run measures the ramp")
     ap.add_argument("--workload", default="c2_interleaved")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
