@@ -150,8 +150,9 @@ struct FwdTraits {
   static constexpr int kThreads = QB * 2;  // QB/32 waves of 64 lanes
   static constexpr int kStep = 64;
   static constexpr int kTileElems = kStep * D;
-  static constexpr size_t kLdsBytes =
-      size_t(2) * 2 * kTileElems * sizeof(uint16_t) + size_t(QB) * 2 * sizeof(uint32_t);
+  // K tiles, V tiles, one pair of mask words per row, 64 mask bytes per row in transit
+  static constexpr size_t kLdsBytes = size_t(2) * 2 * kTileElems * sizeof(uint16_t) +
+                                      size_t(QB) * 2 * sizeof(uint32_t) + size_t(QB) * 64;
 };
 
 // One step of the walk: 64 keys starting at row0, with the effective block mode.
@@ -249,6 +250,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   uint16_t* sK = reinterpret_cast<uint16_t*>(lds_raw);           // [2][TILE]
   uint16_t* sV = sK + 2 * TILE;                                  // [2][TILE]
   uint32_t* sBits = reinterpret_cast<uint32_t*>(sV + 2 * TILE);  // [QB*2]
+  uint8_t* sMaskBytes = reinterpret_cast<uint8_t*>(sBits + QB * 2);  // [QB][64]
 
   // Workgroup -> (slab, query block).  Consecutive workgroup ids go round-robin over
   // the 8 XCDs.  XCD x takes the slabs bh with bh % 8 == x (every batch element's heads
@@ -372,14 +374,26 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     buffer_to_lds_b128(is_v ? rV : rK, is_v ? voff : koff[i % KPER], row * uint32_t(D * 2), dst);
   };
 
-  // PARTIAL blocks: thread tid fetches 32 mask bytes of row tid/2 (a row of its own
-  // wave), packs them to 32 bits and parks the word in LDS for the two lanes that own
-  // the row.  Writer and readers are the same wave, so no workgroup barrier is needed.
-  // Done at the end of the iteration before the one that needs it.
-  auto stage_mask_bits = [&](int it, const StepInfo& si) {
+  // PARTIAL blocks, in two stages so that no load latency is exposed.  One iteration ahead
+  // each wave fetches the 64 mask bytes of its 32 rows for that step straight into LDS (two
+  // buffer->LDS loads per wave, no registers; the resource covers exactly the tile);
+  // at the end of that iteration thread tid packs 32 of the bytes of row tid/2 to 32 bits
+  // and parks the word in LDS for the two lanes that own the row.  Writer and readers of
+  // both stages are the same wave, so no workgroup barrier is needed.
+  auto prefetch_mask_bytes = [&](int it, const StepInfo& si) {
     const int half = it % SPB;
-    const uint8_t* mp = p.partial_masks + size_t(si.pid) * (QB * KB) + size_t(tid >> 1) * KB +
-                        half * STEP + (tid & 1) * 32;
+    const i32x4_t rM = make_buffer_resource(p.partial_masks + size_t(si.pid) * (QB * KB), uint32_t(QB * KB));
+    const uint32_t dst = lds_offset_of(sMaskBytes) + uint32_t(w) * 2048u;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t row = uint32_t(32 * w + 16 * i) + uint32_t(lane >> 2);
+      buffer_to_lds_b128(rM, row * uint32_t(KB) + uint32_t(lane & 3) * 16u, uint32_t(half * STEP),
+                         dst + uint32_t(i) * 1024u);
+    }
+  };
+  auto stage_mask_bits = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the bytes have landed
+    const uint8_t* mp = sMaskBytes + size_t(tid >> 1) * 64 + (tid & 1) * 32;
     const u32x4_t m0 = *reinterpret_cast<const u32x4_t*>(mp);
     const u32x4_t m1 = *reinterpret_cast<const u32x4_t*>(mp + 16);
     uint32_t word = 0;  // byte i (0 or 1) of the 32 -> bit i
@@ -472,12 +486,22 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     }
     kw[0] >>= 4 * g;
     kw[1] >>= 4 * g;
+    // the limit becomes part of the bit words: positions 0 .. lim_l - 32t of word t stay
+    static_for<2>([&](auto tc) {
+      constexpr int t = decltype(tc)::value;
+      const int n = lim_l - 32 * t + 1;  // allowed low positions of word t
+      const uint32_t low = n >= 32 ? 0xffffffffu : (n <= 0 ? 0u : ((1u << (n & 31)) - 1u));
+      kw[t] &= low;
+    });
+    // two instructions per score: the bit, sign-extended to a full word, selects between the
+    // score and -inf
     static_for<32>([&](auto ec) {
       constexpr int e = decltype(ec)::value;
       constexpr int t = e / 16, r = e % 16;
       constexpr int kl = 8 * (r >> 2) + (r & 3);
-      const bool keep = (32 * t + kl <= lim_l) && ((kw[t] >> kl) & 1u);
-      st[SET][t][r] = keep ? st[SET][t][r] : -INFINITY;
+      const uint32_t keep = uint32_t(__builtin_amdgcn_sbfe(int(kw[t]), kl, 1));  // 0 or ~0
+      const uint32_t bits = __builtin_bit_cast(uint32_t, float(st[SET][t][r]));
+      st[SET][t][r] = __builtin_bit_cast(float, (bits & keep) | (0xff800000u & ~keep));
     });
   };
 
@@ -576,7 +600,10 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
       issue_load(NCH + i, 0, cur.row0, 0);
       issue_load(NCH + i, 1, nxt.row0, 0);
     }
-    if (cur.mode == kPartial) stage_mask_bits(0, cur);
+    if (cur.mode == kPartial) {
+      prefetch_mask_bytes(0, cur);
+      stage_mask_bits();
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
 #pragma unroll
@@ -598,8 +625,10 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
       rescale_pending = 0;
     }
     if (!unmasked(cur)) apply_mask(IntC<SET>{}, cur);
+    const bool next_partial = it + 1 < nsteps && nxt.mode == kPartial;
+    if (next_partial) prefetch_mask_bytes(it + 1, nxt);
     body(IntC<SET>{}, first_c, nn.row0, cur.row0);
-    if (it + 1 < nsteps && nxt.mode == kPartial) stage_mask_bits(it + 1, nxt);
+    if (next_partial) stage_mask_bits();
     const StepInfo n3 = step_info(it + 3);
     cur = nxt;
     nxt = nn;
