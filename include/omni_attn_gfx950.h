@@ -47,7 +47,9 @@ enum omni_attn_status {
   OMNI_ATTN_ERR_UNSUPPORTED_BLOCK = 4, /* QB or KB not in {64, 128} */
   OMNI_ATTN_ERR_UNSUPPORTED_DTYPE = 5,
   OMNI_ATTN_ERR_LAUNCH = 6,            /* hipLaunch failed; see omni_attn_last_hip_error() */
-  OMNI_ATTN_ERR_TOO_LARGE = 7          /* a tensor exceeds 2^31-1 elements per (b,h) slab */
+  OMNI_ATTN_ERR_TOO_LARGE = 7,         /* a tensor exceeds 2^31-1 elements per (b,h) slab */
+  OMNI_ATTN_ERR_MISALIGNED = 8         /* q, k, v, o or partial masks not 16-byte aligned, or a
+                                          32-bit array not 4-byte aligned */
 };
 
 /*

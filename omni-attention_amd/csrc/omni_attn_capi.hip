@@ -7,6 +7,7 @@
 #include "omni_attn_fwd_kernel.hpp"
 
 #include <cmath>
+#include <cstdint>
 
 namespace omni_attn {
 template <bool BF16, int D>
@@ -33,6 +34,12 @@ extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v,
   using namespace omni_attn;
   if (!q || !k || !v || !o || !kv_num_blocks || !kv_indices || !block_mask_types)
     return OMNI_ATTN_ERR_NULL_POINTER;
+  // 16-byte loads and stores on q, k, v, o and the mask tiles; 4-byte ones on the rest
+  const auto misaligned = [](const void* ptr, uintptr_t a) { return (reinterpret_cast<uintptr_t>(ptr) & (a - 1)) != 0; };
+  if (misaligned(q, 16) || misaligned(k, 16) || misaligned(v, 16) || misaligned(o, 16) ||
+      misaligned(partial_masks_or_null, 16) || misaligned(lse_or_null, 4) || misaligned(kv_num_blocks, 4) ||
+      misaligned(kv_indices, 4) || misaligned(block_mask_types, 4) || misaligned(partial_idx_or_null, 4))
+    return OMNI_ATTN_ERR_MISALIGNED;
   if (dtype != OMNI_ATTN_DTYPE_F16 && dtype != OMNI_ATTN_DTYPE_BF16)
     return OMNI_ATTN_ERR_UNSUPPORTED_DTYPE;
   if (D != 32 && D != 64 && D != 128) return OMNI_ATTN_ERR_UNSUPPORTED_HEAD_DIM;
@@ -101,6 +108,7 @@ extern "C" const char* omni_attn_status_string(int status) {
     case OMNI_ATTN_ERR_UNSUPPORTED_DTYPE: return "unsupported dtype (supported: fp16, bf16)";
     case OMNI_ATTN_ERR_LAUNCH: return "HIP kernel launch failed";
     case OMNI_ATTN_ERR_TOO_LARGE: return "tensor too large for 32-bit slab indexing";
+    case OMNI_ATTN_ERR_MISALIGNED: return "misaligned pointer: q, k, v, o and partial masks need 16 bytes, 32-bit arrays 4";
     default: return "unknown status";
   }
 }

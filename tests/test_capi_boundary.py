@@ -45,7 +45,8 @@ def test_argument_validation_codes():
     assert call(QB=32) == 4
     assert call(KB=256) == 4
     assert call(dtype=7) == 5
-    for code in range(0, 8):
+    assert call(q=one + 8) == 8     # 16-byte alignment of q, k, v, o
+    for code in range(0, 9):
         assert omni_attn_capi.status_string(code)
     assert "head_dim" in omni_attn_capi.status_string(3)
 
