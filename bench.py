@@ -29,8 +29,8 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs),
 # each scaled by the same counter's reading for a copy kernel of known size; None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    # FETCH_SIZE 199848 KiB x 2.0 (the 256 MiB copy reads 131091) + WRITE_SIZE 66560 KiB x 1.0
-    "c2_interleaved": int((199848 * 2.0 + 66560) * 1024),
+    # FETCH_SIZE 123492 KiB x 2.0 (the 256 MiB copy reads 131091) + WRITE_SIZE 66560 KiB x 1.0
+    "c2_interleaved": int((123492 * 2.0 + 66560) * 1024),
 }
 
 

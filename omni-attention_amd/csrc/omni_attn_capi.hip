@@ -72,15 +72,23 @@ extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v,
   p.n_slabs = B * H;
   // Slabs of one XCD that are walked together, longest query block first.  An XCD has 32
   // CUs and a CU holds two workgroups of this kernel (a Q_BLOCK 64 workgroup is half the
-  // size, four fit): at least enough slabs to fill those slots.  Beyond that, all heads of
+  // size, four fit): at least enough slabs to fill those slots.  Beyond that, the heads of
   // one batch element that land on the XCD (heads of a batch element share their mask in
   // practice, so "query block index" orders their workgroups by length across heads and the
   // tail of one head is filled by the others; mixing batch elements with different masks in
-  // one group measured 8 % slower, a group of one head 2-4 % slower).
+  // one group measured 8 % slower, a group of one head 2-4 % slower) -- but no more heads
+  // than have their K and V in the XCD's 4 MiB L2 together, when at least two do: a bigger
+  // group was 2 % faster still on 4096-token slabs and doubled the L2 misses.
   const int slots_per_xcd = 32 * (QB == 128 ? 2 : 4);
-  const int heads_per_xcd = (H % 8 == 0) ? H / 8 : 1;
   const int fill = slots_per_xcd / Tq > 1 ? slots_per_xcd / Tq : 1;
-  p.slab_group = heads_per_xcd * ((fill + heads_per_xcd - 1) / heads_per_xcd);
+  int heads = (H % 8 == 0) ? H / 8 : 1;
+  const long long slab_kv_bytes = 4LL * S_pad * D;  // K and V, 16-bit
+  const long long fit = (4LL << 20) / slab_kv_bytes;
+  if (fit >= 2 && fit < heads) {
+    heads = int(fit);
+    while ((H / 8) % heads != 0) --heads;  // whole batch elements per group sequence
+  }
+  p.slab_group = heads * ((fill + heads - 1) / heads);
   p.sl2 = float(1.4426950408889634 / std::sqrt(double(D)));
 
   hipStream_t s = static_cast<hipStream_t>(stream);
