@@ -79,6 +79,14 @@ def band_sweep(dev, steps, warmup):
     o = torch.empty_like(q)
     stream = torch.cuda.current_stream(dev)
     points = []
+    # settle the shader clock first (dense mask, some tens of milliseconds of load)
+    nb_w = torch.full((B, H, Tq), Tk, dtype=torch.int32, device=dev)
+    idx_w = torch.arange(Tk, dtype=torch.int32).expand(B, H, Tq, Tk).contiguous().to(dev)
+    tys_w = torch.full((B, H, Tq, Tk), 2, dtype=torch.int32, device=dev)
+    for _ in range(100):
+        omni_attn_capi.fwd(q, k, v, o, None, nb_w, idx_w, tys_w, QB, KB, S, None, None,
+                           stream=stream.cuda_stream)
+    torch.cuda.synchronize()
     w = 1
     while w <= Tk:
         nb = torch.zeros(Tq, dtype=torch.int32)

@@ -203,7 +203,7 @@ def test_runtime_is_linear_in_listed_blocks(gpu_device):
     import bench
 
     r = bench.band_sweep(torch.device(gpu_device), steps=12, warmup=3)
-    assert r["fit"]["r2"] > 0.99, r
+    assert r["fit"]["r2"] > 0.98, r
     assert r["fit"]["ns_per_block"] > 0
 
 
