@@ -237,3 +237,46 @@ def test_wide_score_range_moves_the_reference_often(dtype, gain, gpu_device):
     assert (o32[empty] == 0).all()
     rel_l = ((l32[~empty] - wl[~empty]).abs() / wl[~empty].abs().clamp(min=1.0)).max().item()
     assert rel_l <= TOL_LSE, f"gain {gain}: LSE relative error {rel_l:.3e}"
+
+
+def test_the_forward_can_be_captured_in_a_graph(gpu_device):
+    """No entry point allocates or keeps state: a captured launch replays with new contents
+    of the same buffers.  Replays are interleaved with eager work and synchronisations and
+    every replay is checked against the eager result."""
+    w = make_workload("c3_partial", seed=11, H=2, S=1024)
+    m = w.block_mask
+    dev = gpu_device
+    q, k, v = (t.to(dev).clone() for t in (w.q, w.k, w.v))
+    o = torch.zeros_like(q)
+    lse = torch.zeros(q.shape[:3], dtype=torch.float32, device=dev)
+    nb, idx, tys, pidx, pm = (t.to(dev).contiguous() for t in (m.kv_num_blocks, m.kv_indices, m.block_mask_types,
+                                                                m.partial_block_mask_indices, m.partial_block_masks))
+    S = q.shape[2]
+
+    def launch(stream_ptr=None):
+        omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, pidx, pm,
+                           stream=stream_ptr)
+
+    launch()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(device=dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        launch(side.cuda_stream)  # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            launch(torch.cuda.current_stream(dev).cuda_stream)
+    gen = torch.Generator().manual_seed(5)
+    for rep in range(4):
+        q.copy_(torch.randn(q.shape, generator=gen).to(q.dtype))
+        k.copy_(torch.randn(k.shape, generator=gen).to(k.dtype))
+        torch.cuda.synchronize()
+        o.fill_(float("nan"))
+        lse.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        o_graph, lse_graph = o.clone(), lse.clone()
+        o.fill_(float("nan"))
+        launch()
+        torch.cuda.synchronize()
+        assert torch.equal(o_graph, o) and torch.equal(lse_graph, lse), f"replay {rep}"
