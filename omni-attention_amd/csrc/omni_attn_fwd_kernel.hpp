@@ -15,9 +15,9 @@
 // per-lane scalar.
 //
 // A wave owns 32 query rows; a workgroup has QB/32 waves.  KV blocks are consumed in
-// steps of 64 keys (a 128-key block is two steps).  K and V tiles are double-buffered
-// in LDS and filled by direct buffer->LDS loads (no register staging, out-of-range rows
-// read as zeros).
+// steps of 64 keys (a 128-key block is two steps; 32 keys for 64-row query blocks).  K and
+// V tiles are double-buffered in LDS and filled by direct buffer->LDS loads (no register
+// staging, out-of-range rows read as zeros).
 //
 // The walk is software-pipelined so that the matrix cores and the vector ALU work on
 // different steps inside ONE instruction stream: iteration i of a wave issues the 2*D/16
@@ -148,14 +148,17 @@ __device__ __forceinline__ float pair_sum(float x) {
 template <bool BF16, int D, int QB, int KB>
 struct FwdTraits {
   static constexpr int kThreads = QB * 2;  // QB/32 waves of 64 lanes
-  static constexpr int kStep = 64;
+  // Keys per step.  A 64-row query block has half the waves and would leave LDS room for
+  // only two workgroups per CU (one wave per SIMD) with 64-key tiles: it steps by 32 keys,
+  // four workgroups fit and every SIMD has two waves again.
+  static constexpr int kStep = QB == 64 ? 32 : 64;
   static constexpr int kTileElems = kStep * D;
-  // K tiles, V tiles, one pair of mask words per row, 64 mask bytes per row in transit
+  // K tiles, V tiles, one mask word per row and 32 keys, one mask byte per row and key in transit
   static constexpr size_t kLdsBytes = size_t(2) * 2 * kTileElems * sizeof(uint16_t) +
-                                      size_t(QB) * 2 * sizeof(uint32_t) + size_t(QB) * 64;
+                                      size_t(QB) * (kStep / 32) * sizeof(uint32_t) + size_t(QB) * kStep;
 };
 
-// One step of the walk: 64 keys starting at row0, with the effective block mode.
+// One step of the walk: kStep keys starting at row0, with the effective block mode.
 struct StepInfo {
   int row0;
   int mode;
@@ -239,6 +242,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   constexpr int NT = Traits::kThreads;
   constexpr int STEP = Traits::kStep;
   constexpr int SPB = KB / STEP;        // steps per KV block
+  constexpr int NTL = STEP / 32;        // 32-key accumulator tiles of S^T per step
   constexpr int CPR = D / 8;            // 16-byte chunks per row
   constexpr int NCH = STEP * CPR / NT;  // 16-byte chunks per thread per tile
   constexpr int KS = D / 16;            // MFMA k-steps of Q.K
@@ -249,8 +253,8 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
   uint16_t* sK = reinterpret_cast<uint16_t*>(lds_raw);           // [2][TILE]
   uint16_t* sV = sK + 2 * TILE;                                  // [2][TILE]
-  uint32_t* sBits = reinterpret_cast<uint32_t*>(sV + 2 * TILE);  // [QB*2]
-  uint8_t* sMaskBytes = reinterpret_cast<uint8_t*>(sBits + QB * 2);  // [QB][64]
+  uint32_t* sBits = reinterpret_cast<uint32_t*>(sV + 2 * TILE);  // [QB][NTL]
+  uint8_t* sMaskBytes = reinterpret_cast<uint8_t*>(sBits + QB * NTL);  // [QB][STEP]
 
   // Workgroup -> (slab, query block).  Consecutive workgroup ids go round-robin over
   // the 8 XCDs.  XCD x takes the slabs bh with bh % 8 == x (every batch element's heads
@@ -375,25 +379,29 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   };
 
   // PARTIAL blocks, in two stages so that no load latency is exposed.  One iteration ahead
-  // each wave fetches the 64 mask bytes of its 32 rows for that step straight into LDS (two
-  // buffer->LDS loads per wave, no registers; the resource covers exactly the tile);
-  // at the end of that iteration thread tid packs 32 of the bytes of row tid/2 to 32 bits
-  // and parks the word in LDS for the two lanes that own the row.  Writer and readers of
-  // both stages are the same wave, so no workgroup barrier is needed.
+  // each wave fetches the STEP mask bytes of its 32 rows for that step straight into LDS
+  // (buffer->LDS loads, no registers; the resource covers exactly the tile); at the end of
+  // that iteration a lane packs 32 of the bytes of a row to 32 bits and parks the word in LDS
+  // for the two lanes that own the row.  Writer and readers of both stages are the same wave,
+  // so no workgroup barrier is needed.
+  constexpr int MCPR = STEP / 16;  // 16-byte chunks per row of mask bytes
   auto prefetch_mask_bytes = [&](int it, const StepInfo& si) {
     const int half = it % SPB;
     const i32x4_t rM = make_buffer_resource(p.partial_masks + size_t(si.pid) * (QB * KB), uint32_t(QB * KB));
-    const uint32_t dst = lds_offset_of(sMaskBytes) + uint32_t(w) * 2048u;
+    const uint32_t dst = lds_offset_of(sMaskBytes) + uint32_t(w) * uint32_t(32 * STEP);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const uint32_t row = uint32_t(32 * w + 16 * i) + uint32_t(lane >> 2);
-      buffer_to_lds_b128(rM, row * uint32_t(KB) + uint32_t(lane & 3) * 16u, uint32_t(half * STEP),
+    for (int i = 0; i < MCPR / 2; ++i) {  // 64 / MCPR rows per load
+      const uint32_t row = uint32_t(32 * w + i * (64 / MCPR)) + uint32_t(lane / MCPR);
+      buffer_to_lds_b128(rM, row * uint32_t(KB) + uint32_t(lane % MCPR) * 16u, uint32_t(half * STEP),
                          dst + uint32_t(i) * 1024u);
     }
   };
   auto stage_mask_bits = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the bytes have landed
-    const uint8_t* mp = sMaskBytes + size_t(tid >> 1) * 64 + (tid & 1) * 32;
+    // word NTL * row + h of the wave's 32 rows; with one word per row the upper half-wave
+    // repeats the lower one
+    const int wi = lane % (32 * NTL);
+    const uint8_t* mp = sMaskBytes + size_t(32 * w) * STEP + size_t(wi) * 32;
     const u32x4_t m0 = *reinterpret_cast<const u32x4_t*>(mp);
     const u32x4_t m1 = *reinterpret_cast<const u32x4_t*>(mp + 16);
     uint32_t word = 0;  // byte i (0 or 1) of the 32 -> bit i
@@ -403,10 +411,10 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
       const uint32_t nib = ((bytes & 0x01010101u) * 0x01020408u) >> 24;
       word |= nib << (4 * i);
     }
-    sBits[tid] = word;
+    sBits[32 * w * NTL + wi] = word;
   };
 
-  // Does this wave's 32x64 tile of the step need no mask at all?  (wave-uniform)
+  // Does this wave's 32 x STEP tile of the step need no mask at all?  (wave-uniform)
   auto unmasked = [&](const StepInfo& si) {
     if (si.row0 + STEP > p.seqlen) return false;
     if (si.mode == kFull) return true;
@@ -442,12 +450,12 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   f32x16_t ot[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) ot[dt] = zero16;
-  f32x16_t st[2][2];   // [set][32-key tile]: S^T of the current / next step, alternating
-  u32x4_t pb[2][2][2];  // [set][tile][16-key half]: P^T packed to 16 bits, B-operand order
+  f32x16_t st[2][NTL];   // [set][32-key tile]: S^T of the current / next step, alternating
+  u32x4_t pb[2][NTL][2];  // [set][tile][16-key half]: P^T packed to 16 bits, B-operand order
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < NTL; ++t) {
       st[a][t] = zero16;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) pb[a][t][s2] = u32x4_t{0u, 0u, 0u, 0u};
@@ -463,8 +471,8 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   // SET = it % 2.  Reads K(it+1) from sK[SET^1] into st[SET^1], V(it-1) from sV[SET^1] with
   // pb[SET^1]; softmax of st[SET] into pb[SET]; loads K(it+2) into sK[SET] and V(it) into
   // sV[SET] (both last read one iteration ago).
-  constexpr int NQK = 2 * KS;     // MFMAs of S^T
-  constexpr int NPV_ALL = 4 * DT; // MFMAs of O^T
+  constexpr int NQK = NTL * KS;            // MFMAs of S^T
+  constexpr int NPV_ALL = (STEP / 16) * DT; // MFMAs of O^T
   constexpr int NL = 2 * NCH;     // tile loads per thread
   constexpr int PF_ALL = 3;       // operand fetch distance in slots
   constexpr float kSlack = 6.f;
@@ -478,24 +486,24 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     if (si.mode == kCausal) limit = limit < q_row ? limit : q_row;
     if (si.mode == kMasked) limit = -1;
     const int lim_l = limit - si.row0 - 4 * g;
-    uint32_t kw[2] = {0xffffffffu, 0xffffffffu};
+    uint32_t kw[NTL];
+#pragma unroll
+    for (int t = 0; t < NTL; ++t) kw[t] = 0xffffffffu;
     if (si.mode == kPartial) {
-      const u32x2_t bw = *reinterpret_cast<const u32x2_t*>(sBits + (32 * w + c) * 2);
-      kw[0] = bw[0];
-      kw[1] = bw[1];
+#pragma unroll
+      for (int t = 0; t < NTL; ++t) kw[t] = sBits[(32 * w + c) * NTL + t];
     }
-    kw[0] >>= 4 * g;
-    kw[1] >>= 4 * g;
     // the limit becomes part of the bit words: positions 0 .. lim_l - 32t of word t stay
-    static_for<2>([&](auto tc) {
+    static_for<NTL>([&](auto tc) {
       constexpr int t = decltype(tc)::value;
+      kw[t] >>= 4 * g;
       const int n = lim_l - 32 * t + 1;  // allowed low positions of word t
       const uint32_t low = n >= 32 ? 0xffffffffu : (n <= 0 ? 0u : ((1u << (n & 31)) - 1u));
       kw[t] &= low;
     });
     // two instructions per score: the bit, sign-extended to a full word, selects between the
     // score and -inf
-    static_for<32>([&](auto ec) {
+    static_for<16 * NTL>([&](auto ec) {
       constexpr int e = decltype(ec)::value;
       constexpr int t = e / 16, r = e % 16;
       constexpr int kl = 8 * (r >> 2) + (r & 3);
@@ -513,10 +521,12 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     constexpr int LSP = (NS / 2) / NL > 0 ? (NS / 2) / NL : 1;  // slots between tile loads
     static_assert(NL * LSP <= NS, "tile loads must fit in the slots");
     constexpr int PF = PF_ALL < NS ? PF_ALL : NS;
-    constexpr int NV = 4 + 1 + 16;  // vector chunks: max, reference, 16 exp pairs
+    constexpr int NMX = 2 * NTL;          // max chunks of 8 scores
+    constexpr int NPR = 8 * NTL;          // pairs of exponentials
+    constexpr int NV = NMX + 1 + NPR;     // vector chunks: max, reference, exponentials
     const uint16_t* tK = sK + (SET ^ 1) * TILE;
     const uint16_t* tV = sV + (SET ^ 1) * TILE;
-    auto operand = [&](int n) { return n < NPV ? v_frag(tV, n) : k_frag(tK, (n - NPV) / 2, (n - NPV) % 2); };
+    auto operand = [&](int n) { return n < NPV ? v_frag(tV, n) : k_frag(tK, (n - NPV) / NTL, (n - NPV) % NTL); };
 
     u32x4_t opq[PF];
 #pragma unroll
@@ -526,7 +536,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     auto vector_chunk = [&](auto uc) {
       constexpr int u = decltype(uc)::value;
       if constexpr (u < 0) {
-      } else if constexpr (u < 4) {
+      } else if constexpr (u < NMX) {
         static_for<8>([&](auto ec) {
           constexpr int e = 8 * u + decltype(ec)::value;
           if constexpr ((u & 1) != 0) {
@@ -536,7 +546,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
           }
         });
         pin(mxa, mxb);
-      } else if constexpr (u == 4) {
+      } else if constexpr (u == NMX) {
         // The reference point m_run of the exponentials only has to stay within 2^kSlack of
         // the true running max (P then stays below 2^kSlack, exact in fp32 and well inside
         // the 16-bit types' range), so it is moved -- and O, l rescaled -- only when some
@@ -557,7 +567,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
         rescale_pending |= movers;
         pin(l_run, alpha_pending);
       } else {
-        constexpr int i = u - 5;
+        constexpr int i = u - NMX - 1;
         constexpr int t = i / 8, r = 2 * (i % 8);
         const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[SET][t][r], p.sl2, -m_ref));
         const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[SET][t][r + 1], p.sl2, -m_ref));
@@ -567,7 +577,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
         pin(packed);
         pb[SET][t][r >> 3][(r & 7) >> 1] = packed;
         pin(rs0, rs1);
-        if constexpr (i == 15) l_run += rs0 + rs1;
+        if constexpr (i == NPR - 1) l_run += rs0 + rs1;
       }
     };
 
@@ -577,7 +587,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
         constexpr int ts = j / DT, dt = j % DT;
         ot[dt] = mfma_32x32x16<BF16>(opq[j % PF], pb[SET ^ 1][ts >> 1][ts & 1], ot[dt]);
       } else {
-        constexpr int s = (j - NPV) / 2, t = (j - NPV) % 2;
+        constexpr int s = (j - NPV) / NTL, t = (j - NPV) % NTL;
         st[SET ^ 1][t] = mfma_32x32x16<BF16>(opq[j % PF], qf[s], s == 0 ? zero16 : st[SET ^ 1][t]);
       }
       if constexpr (j + PF < NS) opq[j % PF] = operand(j + PF);
@@ -609,7 +619,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
 #pragma unroll
     for (int s = 0; s < KS; ++s)
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < NTL; ++t)
         st[0][t] = mfma_32x32x16<BF16>(k_frag(sK, s, t), qf[s], s == 0 ? zero16 : st[0][t]);
   }
 
