@@ -7,12 +7,20 @@ Prints ONE JSON line.  `value` is effective TFLOP/s: 4*QB*KB*D flops per listed
 (non-empty) block -- CAUSAL and PARTIAL blocks count as full tiles, softmax flops are
 not counted, EMPTY blocks count nothing -- divided by the wall time per step.
 
+Before the W counted warm-up launches the bench keeps the GPU under this same load for a
+fixed time (--clock-settle-ms, reported as `clock_settle`): from idle the shader clock takes
+some tens of milliseconds of load to reach the level it then holds, and a short run would
+time that ramp instead of the kernel.  K and W are exactly what was passed.
+
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
     python bench.py --sweep-bands     # runtime against the number of listed blocks (fixed shape)
+    python bench.py --kernel-source-hash   # hash that ties a traffic measurement to the kernel sources
 """
 import argparse
+import hashlib
 import json
 import os
+import re
 import statistics
 import sys
 import time
@@ -26,12 +34,77 @@ for _p in (ROOT, PKG):
 METRIC = "effective TFLOP/s (non-empty blocks) + % bf16 MFMA peak, 8K interleaved mask"
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs),
-# each scaled by the same counter's reading for a copy kernel of known size; None = not measured.
-MEASURED_TRAFFIC_BYTES = {
-    # FETCH_SIZE 123492 KiB x 2.0 (the 256 MiB copy reads 131091) + WRITE_SIZE 66560 KiB x 1.0
-    "c2_interleaved": int((123492 * 2.0 + 66560) * 1024),
-}
+# HBM bytes per launch come from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each scaled
+# by what the same counter reads for a plain copy of known size.  The figures live in a tracked
+# summary under profiles/, in a table row per workload that also records the hash of the kernel
+# sources the run was made with; a figure whose hash is not the hash of the sources in this tree
+# describes another kernel and is not reported.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "fwd_kernel_hbm_traffic.md")
+KERNEL_SOURCES = ("omni_attn_fwd_kernel.hpp", "omni_attn_fwd_inst.hip", "omni_attn_capi.hip")
+
+
+def kernel_source_hash() -> str:
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(PKG, "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def read_traffic_profile(path: str = TRAFFIC_PROFILE):
+    """Rows `| workload | FETCH_SIZE KiB | fetch factor | WRITE_SIZE KiB | write factor | hash |`
+    of the tracked summary -> {workload: {"bytes": ..., "kernel_source_hash": ...}}."""
+    out = {}
+    if not os.path.exists(path):
+        return out
+    row = re.compile(r"^\|\s*(\w+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*([0-9a-f]{16})\s*\|")
+    with open(path) as f:
+        for line in f:
+            m = row.match(line)
+            if m:
+                fetch, ff, write, wf = (float(m.group(i)) for i in range(2, 6))
+                out[m.group(1)] = {"bytes": int((fetch * ff + write * wf) * 1024),
+                                   "kernel_source_hash": m.group(6)}
+    return out
+
+
+def traffic_for(workload: str):
+    """(bytes or None, provenance dict) for the roofline object."""
+    rec = read_traffic_profile().get(workload)
+    here = kernel_source_hash()
+    if rec is None:
+        return None, {"source": None, "measured_at_head": False, "kernel_source_hash": here}
+    fresh = rec["kernel_source_hash"] == here
+    return (rec["bytes"] if fresh else None), {
+        "source": os.path.relpath(TRAFFIC_PROFILE, ROOT), "measured_at_head": fresh,
+        "kernel_source_hash": here, "profile_kernel_source_hash": rec["kernel_source_hash"],
+        "stale_bytes": None if fresh else rec["bytes"]}
+
+
+def measure_mfma_peak(dev, dtype_code: int, target_ms: float = 60.0):
+    """TFLOP/s of the library's pure matrix-instruction loop (two waves per SIMD, operands in
+    registers), timed with events on the launch stream after the clock has settled under it."""
+    import torch
+
+    import omni_attn_capi
+
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    iters = 20000
+    t_end = time.perf_counter() + 0.25
+    while time.perf_counter() < t_end:  # settle the clock under this load
+        for _ in range(5):
+            omni_attn_capi.mfma_peak_probe(dtype_code, iters, sink, stream.cuda_stream)
+        torch.cuda.synchronize()
+    best = 0.0
+    for _ in range(5):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        flops = omni_attn_capi.mfma_peak_probe(dtype_code, iters, sink, stream.cuda_stream)
+        b.record(stream)
+        torch.cuda.synchronize()
+        best = max(best, flops / (a.elapsed_time(b) * 1e-3) / 1e12)
+    return best
 
 
 def cpu_baseline(w, budget_s: float):
@@ -137,13 +210,55 @@ def band_sweep(dev, steps, warmup):
     }
 
 
+def extra_workload(name, seed, dev, steps, warmup):
+    """Kernel time of another workload (HIP events on the launch stream, clock already settled)."""
+    import torch
+
+    import omni_attn_capi
+    from baseline_configs import make_workload
+
+    w = make_workload(name, seed=seed)
+    m = w.block_mask
+    B, H, S, D = w.q.shape
+    q, k, v = (t.to(dev) for t in (w.q, w.k, w.v))
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, S, dtype=torch.float32, device=dev)
+    nb, idx, tys = (t.to(dev) for t in (m.kv_num_blocks, m.kv_indices, m.block_mask_types))
+    pidx = None if m.partial_block_mask_indices is None else m.partial_block_mask_indices.to(dev)
+    pm = None if m.partial_block_masks is None else m.partial_block_masks.to(dev)
+    stream = torch.cuda.current_stream(dev)
+
+    def step():
+        omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, pidx, pm,
+                           stream=stream.cuda_stream)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    for i in range(steps):
+        starts[i].record(stream)
+        step()
+        ends[i].record(stream)
+    torch.cuda.synchronize()
+    ms = sum(a.elapsed_time(b) for a, b in zip(starts, ends)) / steps
+    tf = w.effective_flops / (ms * 1e-3) / 1e12
+    return {"workload": f"{name}: B={B} H={H} S={S} D={D}", "nonempty_blocks": w.nonempty_blocks,
+            "kernel_ms_avg": ms, "tflops": tf, "frac": tf / MFMA_PEAK_TFLOPS}
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=100,
-                    help="untimed launches first; the shader clock takes some tens of milliseconds of "
-                         "load to settle, a short run measures the ramp")
+    ap.add_argument("--warmup", type=int, default=100, help="untimed launches before the timed ones")
+    ap.add_argument("--clock-settle-ms", type=float, default=250.0,
+                    help="keep the GPU under the benchmark's own load for this long before the warm-up "
+                         "launches (from idle the shader clock needs some tens of milliseconds to settle)")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the measured MFMA peak and the c2_interleaved_8k figure")
+    ap.add_argument("--kernel-source-hash", action="store_true", help="print the hash and exit")
     ap.add_argument("--workload", default="c2_interleaved")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -154,6 +269,9 @@ def main(argv=None):
     ap.add_argument("--sweep-bands", action="store_true",
                     help="instead of the workload: kernel time against the number of listed blocks")
     args = ap.parse_args(argv)
+    if args.kernel_source_hash:
+        print(kernel_source_hash())
+        return 0
     if args.gpus != 1:
         print("bench.py measures one GPU: (batch, head) slabs are independent, so more GPUs would "
               "only run disjoint slices of the same kernel; run with --gpus 1.", file=sys.stderr)
@@ -189,6 +307,16 @@ def main(argv=None):
         omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, pidx, pm,
                            stream=stream.cuda_stream)
 
+    # clock settle: the same launches, for a fixed time, not counted as warm-up or steps
+    settle_launches = 0
+    t_settle = time.perf_counter()
+    while (time.perf_counter() - t_settle) * 1e3 < args.clock_settle_ms:
+        for _ in range(10):
+            step()
+        settle_launches += 10
+        torch.cuda.synchronize()
+    settle_ms = (time.perf_counter() - t_settle) * 1e3
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -219,6 +347,7 @@ def main(argv=None):
     flops = w.effective_flops
     value = flops / (ms_per_step * 1e-3) / 1e12
     achieved = flops / (avg_kernel_ms * 1e-3) / 1e12
+    traffic, traffic_provenance = traffic_for(args.workload)
 
     out = {
         "metric": METRIC,
@@ -241,6 +370,7 @@ def main(argv=None):
             "total_blocks": B * H * m.num_q_blocks * m.num_kv_blocks,
             "effective_gflop_per_step": flops / 1e9,
         },
+        "clock_settle": {"ms": settle_ms, "launches": settle_launches},
         "pct_of_mfma_peak": 100.0 * value / MFMA_PEAK_TFLOPS,
         "kernel_ms_median": med_kernel_ms,
         "roofline": {
@@ -249,10 +379,19 @@ def main(argv=None):
             "peak": MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / MFMA_PEAK_TFLOPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic": traffic,
+            "traffic_provenance": traffic_provenance,
             "kernel_ms_avg": avg_kernel_ms,
         },
     }
+    if not args.no_extras:
+        dtype_code = omni_attn_capi.DTYPE_BF16 if w.dtype == torch.bfloat16 else omni_attn_capi.DTYPE_F16
+        peak = measure_mfma_peak(dev, dtype_code)
+        out["roofline"]["measured_mfma_peak"] = peak
+        out["roofline"]["frac_of_measured_peak"] = achieved / peak
+        if args.workload == "c2_interleaved":
+            out["c2_interleaved_8k"] = extra_workload("c2_interleaved_8k", args.seed, dev, steps=args.steps,
+                                                      warmup=max(args.warmup, 5))
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, args.cpu_budget_s)
     print(json.dumps(out))

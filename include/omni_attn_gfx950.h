@@ -74,19 +74,24 @@ enum omni_attn_status {
  *   block_mask_types [B, H, Tq, max_blocks] int32, omni_attn_block_type per slot.
  *   partial_idx_or_null   [B, H, Tq, max_blocks] int32 index into partial_masks for
  *                    PARTIAL slots (-1 = none), or NULL when has_partial is false.
- *   partial_masks_or_null [P, QB, KB] one byte per element, 1 = attend, 0 = masked
- *                    (torch.bool storage), row-major q_local*KB + k_local, or NULL.
+ *   partial_masks_or_null [P, QB, KB] one byte per element, non-zero = attend, 0 = masked
+ *                    (torch.bool storage; any non-zero byte counts as attend, as in
+ *                    attn_naive.cu:151), row-major q_local*KB + k_local, or NULL.
+ *   num_partial      P, the number of tiles stored in partial_masks (0 when NULL).  The
+ *                    reference reads tile partial_idx[...] unchecked (attn_naive.cu:124-131);
+ *                    here an index outside [0, P) means "no bits stored".
  *   Tq               number of query blocks, must equal ceil(S_pad / QB).
  *   seqlen_orig      rows >= seqlen_orig are written as zeros (lse -inf); keys
  *                    >= seqlen_orig are never attended (attn_naive.cu:64-72, :113).
  *
  * Semantics per slot: MASKED is skipped; FULL keeps everything; CAUSAL keeps
  * k_global <= q_global; PARTIAL keeps the stored bytes; a PARTIAL slot whose
- * partial pointers are NULL or whose index is negative is skipped
- * (attn_naive.cu:119-131).  A row with no allowed key yields O = 0.
+ * partial pointers are NULL or whose index is negative (attn_naive.cu:119-131) or
+ * >= num_partial is skipped.  A row with no allowed key yields O = 0.
  * The softmax scale is always 1/sqrt(D) (attn_naive.cu:88).
  * Out-of-range metadata cannot fault the device: kv_num_blocks is clamped to
- * [0, max_blocks] and kv_indices to [0, ceil(S_pad / KB) - 1].
+ * [0, max_blocks], kv_indices to [0, ceil(S_pad / KB) - 1], and a partial index outside
+ * [0, num_partial) skips its slot.
  *
  * `stream` is a hipStream_t passed as void* (NULL = the legacy default stream).
  */
@@ -98,8 +103,19 @@ int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v, void* o,
                          const int32_t* partial_idx_or_null,
                          const uint8_t* partial_masks_or_null,
                          int B, int H, int S_pad, int D,
-                         int Tq, int max_blocks, int QB, int KB,
+                         int Tq, int max_blocks, int QB, int KB, int num_partial,
                          int seqlen_orig, int dtype, void* stream);
+
+/*
+ * Measurement aid (no counterpart in the reference): enqueue a kernel that issues nothing but
+ * 32x32x16 matrix instructions of `dtype` from registers -- two workgroups of four waves per
+ * compute unit, `iters` x 8 instructions per wave -- so that a caller timing the launch can
+ * report what the matrix cores of this device sustain at the clock they get under that
+ * load.  *flops_out receives the flop count of the launch; `sink` is a device float the
+ * kernel may write.  Allocates nothing.
+ */
+int omni_attn_mfma_peak_probe_gfx950(int dtype, int iters, float* sink, double* flops_out,
+                                     void* stream);
 
 /* Static description of a return code (never NULL). */
 const char* omni_attn_status_string(int status);
@@ -107,7 +123,7 @@ const char* omni_attn_status_string(int status);
 /* hipError_t of the most recent failed launch on the calling thread (0 if none). */
 int omni_attn_last_hip_error(void);
 
-/* Version of this ABI; bumped when a signature changes. */
+/* Version of this ABI; bumped when a signature changes (2: num_partial added). */
 int omni_attn_abi_version(void);
 
 #ifdef __cplusplus

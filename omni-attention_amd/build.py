@@ -10,11 +10,20 @@ omni-attn-mma/omni_attn_torch.py:548-552):
   libomni_attn_gfx950.so            C ABI (include/omni_attn_gfx950.h), no torch dependency
   omni_attn.cpython-*.so            Python module `omni_attn` (torch tensors in, C ABI underneath)
 
+Every device compile also reports the registers, scratch and occupancy the compiler gave
+each kernel instance (-Rpass-analysis=kernel-resource-usage).  The figures are written to
+build/kernel_resources.json and checked: an instance that spills to scratch memory or
+drops below the waves per SIMD its pipeline is written for fails the build -- the
+instruction schedule of the forward kernel depends on both, and a compiler change would
+otherwise halve the throughput silently.
+
 Usage:  python build.py [--no-ext] [--jobs N]
 """
 import argparse
 import concurrent.futures
+import json
 import os
+import re
 import subprocess
 import sys
 import sysconfig
@@ -30,22 +39,77 @@ HIPCC = os.path.join(ROCM, "bin", "hipcc")
 DEVICE_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-command-line-argument",
+    "-Wno-unused-command-line-argument", "-Wno-inline-asm",
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+RESOURCES_JSON = os.path.join(OBJ, "kernel_resources.json")
+
+# What every kernel of the library must keep: no scratch memory, no spilled registers, and
+# at least this many waves per SIMD (kernels are matched by a substring of their mangled name).
+MIN_WAVES_PER_SIMD = {"fwd_kernel": 2}
 
 INSTANCES = [(bf, d) for bf in (0, 1) for d in (32, 64, 128)]
 LIB_NAME = "libomni_attn_gfx950.so"
 
 
+_REMARK = re.compile(r"remark:\s+(Function Name|TotalSGPRs|VGPRs|AGPRs|ScratchSize \[bytes/lane\]|"
+                     r"Occupancy \[waves/SIMD\]|SGPRs Spill|VGPRs Spill|LDS Size \[bytes/block\]):\s+(\S+)")
+_KEYS = {"TotalSGPRs": "sgprs", "VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch_bytes",
+         "Occupancy [waves/SIMD]": "waves_per_simd", "SGPRs Spill": "sgpr_spills", "VGPRs Spill": "vgpr_spills",
+         "LDS Size [bytes/block]": "static_lds_bytes"}
+
+
+def parse_resource_remarks(text):
+    """Compiler remarks of one device compile -> {mangled kernel name: {figure: value}}."""
+    kernels, cur = {}, None
+    for line in text.splitlines():
+        m = _REMARK.search(line)
+        if not m:
+            continue
+        key, val = m.group(1), m.group(2)
+        if key == "Function Name":
+            cur = kernels.setdefault(val, {})
+        elif cur is not None:
+            cur[_KEYS[key]] = int(val)
+    return kernels
+
+
+def check_resources(kernels):
+    """Raise if a kernel uses scratch memory, spills, or falls below its waves per SIMD."""
+    problems = []
+    for name, r in sorted(kernels.items()):
+        if r.get("scratch_bytes", 0) or r.get("vgpr_spills", 0) or r.get("sgpr_spills", 0):
+            problems.append("%s: scratch %d B/lane, %d VGPR / %d SGPR spills" % (
+                name, r.get("scratch_bytes", 0), r.get("vgpr_spills", 0), r.get("sgpr_spills", 0)))
+        for pattern, waves in MIN_WAVES_PER_SIMD.items():
+            if pattern in name and r.get("waves_per_simd", 0) < waves:
+                problems.append("%s: %d waves per SIMD, needs %d (%d VGPRs, %d AGPRs)" % (
+                    name, r.get("waves_per_simd", 0), waves, r.get("vgprs", -1), r.get("agprs", -1)))
+    if problems:
+        raise RuntimeError("kernel resource check failed:\n  " + "\n  ".join(problems))
+
+
 def _run(cmd):
+    """Run a compiler command; returns (diagnostics without the resource remarks, remarks)."""
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(
-        line for line in proc.stdout.splitlines()
-        if "packed-fp32-ops' is not a recognized feature" not in line
-    )
+    lines = proc.stdout.splitlines()
+    remarks = "\n".join(l for l in lines if "-Rpass-analysis=kernel-resource-usage" in l)
+    keep, skip = [], 0
+    for l in lines:
+        if "-Rpass-analysis=kernel-resource-usage" in l:
+            skip = 2  # the source line and caret that follow a remark
+            continue
+        if skip and (re.match(r"^\s*\d+ \|", l) or re.match(r"^\s*\|?\s*\^", l)):
+            skip -= 1
+            continue
+        skip = 0
+        if "packed-fp32-ops' is not a recognized feature" in l or "In file included from" in l:
+            continue
+        keep.append(l)
+    out = "\n".join(keep)
     if proc.returncode != 0:
-        raise RuntimeError("command failed (%d): %s\n%s" % (proc.returncode, " ".join(cmd), out))
-    return out
+        raise RuntimeError("command failed (%d): %s\n%s" % (proc.returncode, " ".join(cmd), proc.stdout))
+    return out, remarks
 
 
 def build_capi(jobs):
@@ -58,13 +122,19 @@ def build_capi(jobs):
         cmds.append([HIPCC] + DEVICE_FLAGS + [
             "-DOMNI_INST_BF16=%d" % bf, "-DOMNI_INST_D=%d" % d,
             "-c", os.path.join(CSRC, "omni_attn_fwd_inst.hip"), "-o", obj])
-    obj = os.path.join(OBJ, "omni_attn_capi.o")
-    objs.append(obj)
-    cmds.append([HIPCC] + DEVICE_FLAGS + ["-c", os.path.join(CSRC, "omni_attn_capi.hip"), "-o", obj])
+    for src in ("omni_attn_capi", "omni_attn_probe"):
+        obj = os.path.join(OBJ, src + ".o")
+        objs.append(obj)
+        cmds.append([HIPCC] + DEVICE_FLAGS + ["-c", os.path.join(CSRC, src + ".hip"), "-o", obj])
+    kernels = {}
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        for out in pool.map(_run, cmds):
+        for out, remarks in pool.map(_run, cmds):
             if out.strip():
                 print(out)
+            kernels.update(parse_resource_remarks(remarks))
+    with open(RESOURCES_JSON, "w") as f:
+        json.dump(kernels, f, indent=1, sort_keys=True)
+    check_resources(kernels)
     lib = os.path.join(HERE, LIB_NAME)
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs)
     return lib

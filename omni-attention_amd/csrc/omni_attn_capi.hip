@@ -6,6 +6,7 @@
 #include "../../include/omni_attn_gfx950.h"
 #include "omni_attn_fwd_kernel.hpp"
 
+#include <atomic>
 #include <cmath>
 #include <cstdint>
 
@@ -22,15 +23,54 @@ template <> int launch_fwd_blocks<true, 128>(const FwdParams&, int, int, hipStre
 
 namespace {
 thread_local int g_last_hip_error = 0;
+
+// What the work order needs to know about the device, queried once per device: the number
+// of XCDs (each has its own L2; workgroup ids are dealt round-robin over them), the compute
+// units per XCD and the size of one L2.  A partitioned device (CPX: one XCD per device)
+// reports 1 XCD and its own CU count.
+struct DeviceTopology {
+  int n_xcd;
+  int cus_per_xcd;
+  long long l2_bytes;
+};
+constexpr int kMaxDevices = 64;
+DeviceTopology g_topology[kMaxDevices];
+std::atomic<bool> g_topology_known[kMaxDevices];
+
+int query_topology(DeviceTopology* out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return int(e);
+  const bool cached = dev >= 0 && dev < kMaxDevices;
+  if (cached && g_topology_known[dev].load(std::memory_order_acquire)) {
+    *out = g_topology[dev];
+    return 0;
+  }
+  int xcc = 0, cus = 0, l2 = 0;
+  if (hipDeviceGetAttribute(&xcc, hipDeviceAttributeNumberOfXccs, dev) != hipSuccess || xcc <= 0) xcc = 1;
+  e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e != hipSuccess) return int(e);
+  if (hipDeviceGetAttribute(&l2, hipDeviceAttributeL2CacheSize, dev) != hipSuccess || l2 <= 0) l2 = 4 << 20;
+  DeviceTopology t;
+  t.n_xcd = xcc;
+  t.cus_per_xcd = cus / xcc > 0 ? cus / xcc : 1;
+  t.l2_bytes = l2;
+  if (cached) {
+    g_topology[dev] = t;
+    g_topology_known[dev].store(true, std::memory_order_release);
+  }
+  *out = t;
+  return 0;
 }
+}  // namespace
 
 extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v, void* o,
                                     float* lse_or_null, const int32_t* kv_num_blocks,
                                     const int32_t* kv_indices, const int32_t* block_mask_types,
                                     const int32_t* partial_idx_or_null,
                                     const uint8_t* partial_masks_or_null, int B, int H, int S_pad,
-                                    int D, int Tq, int max_blocks, int QB, int KB, int seqlen_orig,
-                                    int dtype, void* stream) {
+                                    int D, int Tq, int max_blocks, int QB, int KB, int num_partial,
+                                    int seqlen_orig, int dtype, void* stream) {
   using namespace omni_attn;
   if (!q || !k || !v || !o || !kv_num_blocks || !kv_indices || !block_mask_types)
     return OMNI_ATTN_ERR_NULL_POINTER;
@@ -44,7 +84,7 @@ extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v,
     return OMNI_ATTN_ERR_UNSUPPORTED_DTYPE;
   if (D != 32 && D != 64 && D != 128) return OMNI_ATTN_ERR_UNSUPPORTED_HEAD_DIM;
   if ((QB != 64 && QB != 128) || (KB != 64 && KB != 128)) return OMNI_ATTN_ERR_UNSUPPORTED_BLOCK;
-  if (B <= 0 || H <= 0 || S_pad <= 0 || Tq <= 0 || max_blocks <= 0 || seqlen_orig < 0)
+  if (B <= 0 || H <= 0 || S_pad <= 0 || Tq <= 0 || max_blocks <= 0 || seqlen_orig < 0 || num_partial < 0)
     return OMNI_ATTN_ERR_BAD_SHAPE;
   if (Tq != (S_pad + QB - 1) / QB) return OMNI_ATTN_ERR_BAD_SHAPE;
   const long long total = (long long)B * H * Tq;
@@ -61,32 +101,41 @@ extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v,
   p.kv_num_blocks = kv_num_blocks;
   p.kv_indices = kv_indices;
   p.types = block_mask_types;
-  const bool has_partial = partial_idx_or_null != nullptr && partial_masks_or_null != nullptr;
+  if ((long long)num_partial * QB * KB > 0x7fffffffLL * 64) return OMNI_ATTN_ERR_TOO_LARGE;
+  const bool has_partial = partial_idx_or_null != nullptr && partial_masks_or_null != nullptr && num_partial > 0;
   p.partial_idx = has_partial ? partial_idx_or_null : nullptr;
   p.partial_masks = has_partial ? partial_masks_or_null : nullptr;
+  p.num_partial = has_partial ? num_partial : 0;
   p.S = S_pad;
   p.Tq = Tq;
   p.Tk = (S_pad + KB - 1) / KB;
   p.max_blocks = max_blocks;
   p.seqlen = seqlen_orig < S_pad ? seqlen_orig : S_pad;
   p.n_slabs = B * H;
-  // Slabs of one XCD that are walked together, longest query block first.  An XCD has 32
-  // CUs and a CU holds two workgroups of this kernel (a Q_BLOCK 64 workgroup is half the
-  // size, four fit): at least enough slabs to fill those slots.  Beyond that, the heads of
+  DeviceTopology topo;
+  if (const int e = query_topology(&topo)) {
+    g_last_hip_error = e;
+    return OMNI_ATTN_ERR_LAUNCH;
+  }
+  p.n_xcd = topo.n_xcd;
+  const int X = topo.n_xcd;
+  // Slabs of one XCD that are walked together, longest query block first.  A CU holds two
+  // workgroups of this kernel (a Q_BLOCK 64 workgroup is half the size, four fit): at
+  // least enough slabs to fill the XCD's slots.  Beyond that, the heads of
   // one batch element that land on the XCD (heads of a batch element share their mask in
   // practice, so "query block index" orders their workgroups by length across heads and the
   // tail of one head is filled by the others; mixing batch elements with different masks in
   // one group measured 8 % slower, a group of one head 2-4 % slower) -- but no more heads
-  // than have their K and V in the XCD's 4 MiB L2 together, when at least two do: a bigger
-  // group was 2 % faster still on 4096-token slabs and doubled the L2 misses.
-  const int slots_per_xcd = 32 * (QB == 128 ? 2 : 4);
+  // than have their K and V in the XCD's L2 (4 MiB on MI355X) together, when at least two
+  // do: a bigger group was 2 % faster still on 4096-token slabs and doubled the L2 misses.
+  const int slots_per_xcd = topo.cus_per_xcd * (QB == 128 ? 2 : 4);
   const int fill = slots_per_xcd / Tq > 1 ? slots_per_xcd / Tq : 1;
-  int heads = (H % 8 == 0) ? H / 8 : 1;
+  int heads = (H % X == 0) ? H / X : 1;
   const long long slab_kv_bytes = 4LL * S_pad * D;  // K and V, 16-bit
-  const long long fit = (4LL << 20) / slab_kv_bytes;
+  const long long fit = topo.l2_bytes / slab_kv_bytes;
   if (fit >= 2 && fit < heads) {
     heads = int(fit);
-    while ((H / 8) % heads != 0) --heads;  // whole batch elements per group sequence
+    while ((H / X) % heads != 0) --heads;  // whole batch elements per group sequence
   }
   p.slab_group = heads * ((fill + heads - 1) / heads);
   p.sl2 = float(1.4426950408889634 / std::sqrt(double(D)));
@@ -123,4 +172,4 @@ extern "C" const char* omni_attn_status_string(int status) {
 
 extern "C" int omni_attn_last_hip_error(void) { return g_last_hip_error; }
 
-extern "C" int omni_attn_abi_version(void) { return 1; }
+extern "C" int omni_attn_abi_version(void) { return 2; }

@@ -36,6 +36,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <utility>
 
 namespace omni_attn {
@@ -62,12 +63,14 @@ struct FwdParams {
   const int32_t* types;          // [B,H,Tq,max_blocks]
   const int32_t* partial_idx;    // [B,H,Tq,max_blocks] or null
   const uint8_t* partial_masks;  // [P,QB,KB] bytes or null
+  int num_partial; // P: tiles stored in partial_masks
   int S;           // padded sequence length (rows per (b,h) slab)
   int Tq;          // query blocks per slab
   int Tk;          // ceil(S / KB)
   int max_blocks;  // slots per query block
   int seqlen;      // min(seqlen_orig, S): rows/keys at or beyond it are padding
   int n_slabs;     // B*H
+  int n_xcd;       // XCDs (L2 domains) of the device; workgroup ids go round-robin over them
   int slab_group;  // slabs of one XCD that are walked together (>= 1)
   float sl2;       // log2(e) / sqrt(D)
 };
@@ -257,7 +260,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   uint8_t* sMaskBytes = reinterpret_cast<uint8_t*>(sBits + QB * NTL);  // [QB][STEP]
 
   // Workgroup -> (slab, query block).  Consecutive workgroup ids go round-robin over
-  // the 8 XCDs.  XCD x takes the slabs bh with bh % 8 == x (every batch element's heads
+  // the XCDs.  XCD x takes the slabs bh with bh % n_xcd == x (every batch element's heads
   // are spread over all XCDs, which balances batches with different masks) and works
   // through them in groups of p.slab_group slabs, sized so that one group's query
   // blocks just fill the XCD's workgroup slots: the workgroups that run together then
@@ -266,9 +269,9 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   // query blocks.  Inside a group the order is longest-first: query block Tq-1 of each
   // slab of the group, then Tq-2, ...
   const int wg = blockIdx.x;
-  const int xcd = wg & 7;
-  const int slot = wg >> 3;
-  const int slabs_here = (p.n_slabs - xcd + 7) >> 3;
+  const int slot = wg / p.n_xcd;
+  const int xcd = wg - slot * p.n_xcd;
+  const int slabs_here = (p.n_slabs - xcd + p.n_xcd - 1) / p.n_xcd;
   if (slot >= slabs_here * p.Tq) return;
   const int per_group = p.slab_group * p.Tq;
   const int gi = slot / per_group;
@@ -276,7 +279,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   const int g_left = slabs_here - gi * p.slab_group;
   const int g_eff = g_left < p.slab_group ? g_left : p.slab_group;
   const int qrank = in_group / g_eff;
-  const int bh = xcd + 8 * (gi * p.slab_group + (in_group - qrank * g_eff));
+  const int bh = xcd + p.n_xcd * (gi * p.slab_group + (in_group - qrank * g_eff));
   const int qb = p.Tq - 1 - qrank;
 
   const int tid = threadIdx.x;
@@ -312,7 +315,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     const int32_t pid = has_partial ? p.partial_idx[o] : -1;
     const int32_t kvb = kvb_raw < 0 ? 0 : (kvb_raw >= p.Tk ? p.Tk - 1 : kvb_raw);
     int32_t mode = (ty == kCausal || ty == kFull || ty == kPartial) ? ty : int32_t(kMasked);
-    if (ty == kPartial && pid < 0) mode = kMasked;
+    if (ty == kPartial && (pid < 0 || pid >= p.num_partial)) mode = kMasked;
     mv_row0 = kvb * KB;
     mv_mode = mode;
     mv_pid = pid;
@@ -404,10 +407,13 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     const uint8_t* mp = sMaskBytes + size_t(32 * w) * STEP + size_t(wi) * 32;
     const u32x4_t m0 = *reinterpret_cast<const u32x4_t*>(mp);
     const u32x4_t m1 = *reinterpret_cast<const u32x4_t*>(mp + 16);
-    uint32_t word = 0;  // byte i (0 or 1) of the 32 -> bit i
+    uint32_t word = 0;  // byte i of the 32 (any non-zero value = attend, attn_naive.cu:151) -> bit i
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const uint32_t bytes = i < 4 ? m0[i] : m1[i - 4];
+      uint32_t bytes = i < 4 ? m0[i] : m1[i - 4];
+      bytes |= bytes >> 4;  // fold each byte onto its lowest bit
+      bytes |= bytes >> 2;
+      bytes |= bytes >> 1;
       const uint32_t nib = ((bytes & 0x01010101u) * 0x01020408u) >> 24;
       word |= nib << (4 * i);
     }
@@ -717,20 +723,32 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   }
 }
 
-// Host-side launch of one instance; returns the hipError_t of the launch.
+// Host-side launch of one instance; returns the hipError_t of the launch itself (the
+// thread's sticky "last error" of earlier, unrelated HIP calls is neither read nor cleared).
+// The dynamic-LDS limit of an instance is raised once per device, not on every launch.
+constexpr int kMaxDevices = 64;
 template <bool BF16, int D, int QB, int KB>
 int launch_fwd(const FwdParams& p, hipStream_t stream) {
   using Traits = FwdTraits<BF16, D, QB, KB>;
   auto kern = fwd_kernel<BF16, D, QB, KB>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     int(Traits::kLdsBytes));
+  static std::atomic<bool> lds_limit_set[kMaxDevices];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return int(e);
-  const unsigned slabs_per_xcd = unsigned(p.n_slabs + 7) / 8u;
-  const dim3 grid(8u * slabs_per_xcd * unsigned(p.Tq));
+  const bool cached = dev >= 0 && dev < kMaxDevices;
+  if (!cached || !lds_limit_set[dev].load(std::memory_order_acquire)) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, int(Traits::kLdsBytes));
+    if (e != hipSuccess) return int(e);
+    if (cached) lds_limit_set[dev].store(true, std::memory_order_release);
+  }
+  const unsigned slabs_per_xcd = unsigned(p.n_slabs + p.n_xcd - 1) / unsigned(p.n_xcd);
+  const dim3 grid(unsigned(p.n_xcd) * slabs_per_xcd * unsigned(p.Tq));
   const dim3 block(Traits::kThreads);
-  hipLaunchKernelGGL(kern, grid, block, Traits::kLdsBytes, stream, p);
-  return int(hipGetLastError());
+  FwdParams params = p;
+  void* args[] = {&params};
+  return int(hipLaunchKernel(reinterpret_cast<const void*>(kern), grid, block, args,
+                             Traits::kLdsBytes, stream));
 }
 
 }  // namespace omni_attn

@@ -81,6 +81,7 @@ void forward_impl(const torch::Tensor& Q, const torch::Tensor& K, const torch::T
 
   const int32_t* pidx = nullptr;
   const uint8_t* pmask = nullptr;
+  int num_partial = 0;
   if (has_partial) {
     if (partial_block_mask_indices.scalar_type() != torch::kInt32)
       throw std::runtime_error(
@@ -101,6 +102,7 @@ void forward_impl(const torch::Tensor& Q, const torch::Tensor& K, const torch::T
     if (partial_block_masks.size(0) > 0) {
       pidx = partial_block_mask_indices.data_ptr<int32_t>();
       pmask = reinterpret_cast<const uint8_t*>(partial_block_masks.data_ptr<bool>());
+      num_partial = int(partial_block_masks.size(0));
     }
   }
 
@@ -111,7 +113,7 @@ void forward_impl(const torch::Tensor& Q, const torch::Tensor& K, const torch::T
       Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), lse,
       kv_num_blocks.data_ptr<int32_t>(), kv_indices.data_ptr<int32_t>(),
       block_mask_types.data_ptr<int32_t>(), pidx, pmask, int(B), int(H), int(S), int(D),
-      int(num_q_blocks), int(max_blocks), Q_BLOCK_SIZE, KV_BLOCK_SIZE, seqlen_orig, dtype,
+      int(num_q_blocks), int(max_blocks), Q_BLOCK_SIZE, KV_BLOCK_SIZE, num_partial, seqlen_orig, dtype,
       static_cast<void*>(stream));
   if (rc != OMNI_ATTN_OK) {
     std::string msg = std::string("omni_attn: ") + omni_attn_status_string(rc);

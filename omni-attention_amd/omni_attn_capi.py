@@ -19,6 +19,7 @@ DTYPE_BF16 = 1
 
 EXPORTED_SYMBOLS = (
     "omni_attn_fwd_gfx950",
+    "omni_attn_mfma_peak_probe_gfx950",
     "omni_attn_status_string",
     "omni_attn_last_hip_error",
     "omni_attn_abi_version",
@@ -33,7 +34,9 @@ def load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(LIB_PATH)
         vp, i32 = ctypes.c_void_p, ctypes.c_int
         lib.omni_attn_fwd_gfx950.restype = i32
-        lib.omni_attn_fwd_gfx950.argtypes = [vp] * 10 + [i32] * 10 + [vp]
+        lib.omni_attn_fwd_gfx950.argtypes = [vp] * 10 + [i32] * 11 + [vp]
+        lib.omni_attn_mfma_peak_probe_gfx950.restype = i32
+        lib.omni_attn_mfma_peak_probe_gfx950.argtypes = [i32, i32, vp, ctypes.POINTER(ctypes.c_double), vp]
         lib.omni_attn_status_string.restype = ctypes.c_char_p
         lib.omni_attn_status_string.argtypes = [i32]
         lib.omni_attn_last_hip_error.restype = i32
@@ -46,16 +49,28 @@ def status_string(code: int) -> str:
     return load_library().omni_attn_status_string(int(code)).decode()
 
 
+def mfma_peak_probe(dtype: int, iters: int, sink: torch.Tensor, stream: Optional[int] = None) -> float:
+    """Enqueue the pure matrix-instruction loop; returns the flop count of the launch."""
+    flops = ctypes.c_double(0.0)
+    if stream is None:
+        stream = torch.cuda.current_stream(sink.device).cuda_stream
+    with torch.cuda.device(sink.device):
+        rc = load_library().omni_attn_mfma_peak_probe_gfx950(dtype, iters, sink.data_ptr(), ctypes.byref(flops), stream)
+    if rc != 0:
+        raise RuntimeError("omni_attn_mfma_peak_probe_gfx950: %s (status %d)" % (status_string(rc), rc))
+    return flops.value
+
+
 def _ptr(t: Optional[torch.Tensor]) -> int:
     return 0 if t is None else t.data_ptr()
 
 
 def fwd_raw(q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, nb_ptr, idx_ptr, types_ptr, pidx_ptr, pmask_ptr,
-            B, H, S_pad, D, Tq, max_blocks, QB, KB, seqlen_orig, dtype, stream_ptr) -> int:
+            B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial, seqlen_orig, dtype, stream_ptr) -> int:
     """The C call itself; returns the status code."""
     return load_library().omni_attn_fwd_gfx950(
         q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, nb_ptr, idx_ptr, types_ptr, pidx_ptr, pmask_ptr,
-        B, H, S_pad, D, Tq, max_blocks, QB, KB, seqlen_orig, dtype, stream_ptr)
+        B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial, seqlen_orig, dtype, stream_ptr)
 
 
 def fwd(q, k, v, o, lse, kv_num_blocks, kv_indices, block_mask_types, QB, KB, seqlen_orig,
@@ -88,6 +103,7 @@ def fwd(q, k, v, o, lse, kv_num_blocks, kv_indices, block_mask_types, QB, KB, se
         rc = fwd_raw(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(kv_num_blocks),
                      _ptr(kv_indices), _ptr(block_mask_types), _ptr(partial_idx), _ptr(partial_masks),
                      B, H, S, D, kv_num_blocks.shape[2], kv_indices.shape[3], QB, KB,
+                     0 if partial_masks is None else int(partial_masks.shape[0]),
                      int(seqlen_orig), dtype, stream)
     if rc != 0:
         raise RuntimeError("omni_attn_fwd_gfx950: %s (status %d)" % (status_string(rc), rc))

@@ -25,8 +25,8 @@ static int imin(int a, int b) { return a < b ? a : b; }
 /* Visit every allowed key of row q_idx; pass 0 finds the max, pass 1 accumulates. */
 static void walk_row(const float* Q, const float* K, const float* V, float* out, float* max_score,
                      float* sum_exp, int pass, const int32_t* kv_indices, const int32_t* types,
-                     const int32_t* partial_idx, const uint8_t* partial_masks, int kv_nb,
-                     int q_idx, int q_block, int QB, int KB, int seqlen_orig, int D) {
+                     const int32_t* partial_idx, const uint8_t* partial_masks, int num_partial,
+                     int kv_nb, int q_idx, int q_block, int QB, int KB, int seqlen_orig, int D) {
   const float scale = 1.0f / sqrtf((float)D); /* attn_naive.cu:88 */
   const float* qrow = Q + (size_t)q_idx * D;
   for (int s = 0; s < kv_nb; ++s) {
@@ -43,6 +43,9 @@ static void walk_row(const float* Q, const float* K, const float* V, float* out,
       if (!partial_idx || !partial_masks) continue;
       pid = partial_idx[s];
       if (pid < 0) continue;
+      /* the reference reads any index unchecked; the product's contract is that an index
+       * beyond the stored tiles means "no bits stored", like a negative one */
+      if (pid >= num_partial) continue;
     }
     if (mask_type == BLOCK_MASK_CAUSAL) { /* :134-140 */
       if (q_idx < kv_start) continue;
@@ -79,7 +82,7 @@ int omni_oracle_block_walk(const float* q, const float* k, const float* v, float
                            const int32_t* kv_num_blocks, const int32_t* kv_indices,
                            const int32_t* block_mask_types, const int32_t* partial_idx,
                            const uint8_t* partial_masks, int B, int H, int S, int D, int Tq,
-                           int max_blocks, int QB, int KB, int seqlen_orig) {
+                           int max_blocks, int QB, int KB, int num_partial, int seqlen_orig) {
   if (!q || !k || !v || !o || !lse || !kv_num_blocks || !kv_indices || !block_mask_types) return -1;
   if (B <= 0 || H <= 0 || S <= 0 || D <= 0 || D > 256 || Tq <= 0 || max_blocks <= 0) return -1;
   if (seqlen_orig > S) seqlen_orig = S;
@@ -105,10 +108,10 @@ int omni_oracle_block_walk(const float* q, const float* k, const float* v, float
     float acc[256];
     for (int d = 0; d < D; ++d) acc[d] = 0.0f;
     walk_row(q + slab, k + slab, v + slab, acc, &max_score, &sum_exp, 0, idx, tys, pidx,
-             partial_masks, kv_nb, q_idx, q_block, QB, KB, seqlen_orig, D);
+             partial_masks, num_partial, kv_nb, q_idx, q_block, QB, KB, seqlen_orig, D);
     if (max_score == -INFINITY) continue; /* everything masked: zeros, :177-183 */
     walk_row(q + slab, k + slab, v + slab, acc, &max_score, &sum_exp, 1, idx, tys, pidx,
-             partial_masks, kv_nb, q_idx, q_block, QB, KB, seqlen_orig, D);
+             partial_masks, num_partial, kv_nb, q_idx, q_block, QB, KB, seqlen_orig, D);
     if (sum_exp <= 0.0f) continue; /* :283-288 */
     const float inv = 1.0f / sum_exp;
     for (int d = 0; d < D; ++d) orow[d] = acc[d] * inv;

@@ -44,6 +44,7 @@ def attention_block_walk(q, k, v, kv_num_blocks, kv_indices, block_mask_types, Q
     rc = lib.omni_oracle_block_walk(_ptr(qf), _ptr(kf), _ptr(vf), _ptr(o), _ptr(lse), _ptr(nb),
                                     _ptr(idx), _ptr(tys), _ptr(pidx), _ptr(pm), B, H, S, D,
                                     nb.shape[2], idx.shape[3], QB, KB,
+                                    0 if pm is None else int(pm.shape[0]),
                                     S if seqlen_orig is None else int(seqlen_orig))
     if rc != 0:
         raise RuntimeError("omni_oracle_block_walk failed with %d" % rc)

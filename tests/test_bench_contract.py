@@ -17,6 +17,33 @@ def test_more_than_one_gpu_is_refused_with_a_message():
     assert "one GPU" in r.stderr and r.stdout.strip() == ""
 
 
+def test_traffic_figure_comes_from_the_tracked_profile_and_is_tied_to_the_kernel_sources(tmp_path):
+    sys.path.insert(0, ROOT)
+    import bench
+    rows = bench.read_traffic_profile()
+    assert "c2_interleaved" in rows
+    text = open(bench.TRAFFIC_PROFILE).read()
+    for name, rec in rows.items():
+        line = next(ln for ln in text.splitlines() if ln.startswith("| " + name + " "))
+        cells = [c.strip() for c in line.strip("|").split("|")]
+        assert rec["bytes"] == int((float(cells[1]) * float(cells[2]) + float(cells[3]) * float(cells[4])) * 1024)
+        assert rec["kernel_source_hash"] == cells[5]
+        # compulsory bytes of c2: Q, K, V, O of [2, 32, 4096, 128] 16-bit: the counters cannot show less
+        if name == "c2_interleaved":
+            assert rec["bytes"] >= 4 * 2 * 32 * 4096 * 128 * 2
+    value, prov = bench.traffic_for("c2_interleaved")
+    assert prov["kernel_source_hash"] == bench.kernel_source_hash()
+    if prov["measured_at_head"]:
+        assert value == rows["c2_interleaved"]["bytes"]
+    else:
+        assert value is None and prov["stale_bytes"] == rows["c2_interleaved"]["bytes"]
+    assert bench.traffic_for("no_such_workload")[0] is None
+    # a row with another hash is never reported
+    p = tmp_path / "t.md"
+    p.write_text("| c2_interleaved | 10 | 2.0 | 5 | 1.0 | 0123456789abcdef |\n")
+    assert bench.read_traffic_profile(str(p))["c2_interleaved"]["bytes"] == 25 * 1024
+
+
 @pytest.mark.gpu
 def test_json_line_has_the_contract_fields(gpu_device):
     r = subprocess.run([sys.executable, BENCH, "--workload", "c1_causal", "--steps", "5", "--warmup", "2",
@@ -29,10 +56,12 @@ def test_json_line_has_the_contract_fields(gpu_device):
                 "scaling", "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
         assert key in d, key
     assert d["n_gpus"] == 1 and d["steps"] == 5 and d["warmup"] == 2 and d["vs_baseline"] is None
+    assert d["clock_settle"]["launches"] > 0 and d["clock_settle"]["ms"] >= 250.0
     assert d["unit"] == "TFLOP/s" and d["dtype"] in ("bf16", "f16") and d["data"] == "synthetic"
     assert "workload" in d["config"] and "model" not in d["config"]
     rf = d["roofline"]
     assert rf["bound"] == "mfma" and rf["unit"] == "TFLOP/s" and rf["peak"] == 2500.0
     assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-12 and "traffic" in rf
+    assert 500.0 < rf["measured_mfma_peak"] < 2600.0 and "measured_at_head" in rf["traffic_provenance"]
     cb = d["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]

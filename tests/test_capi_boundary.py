@@ -28,18 +28,19 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(omni_attn_capi.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert omni_attn_capi.load_library().omni_attn_abi_version() == 1
+    assert omni_attn_capi.load_library().omni_attn_abi_version() == 2
 
 
 def test_argument_validation_codes():
     lib = omni_attn_capi.load_library()
     one = 4096  # any non-null value: validation fails before it would be dereferenced
-    def call(q=one, D=128, QB=128, KB=128, Tq=4, S=512, dtype=1, B=1):
+    def call(q=one, D=128, QB=128, KB=128, Tq=4, S=512, dtype=1, B=1, P=0):
         return omni_attn_capi.fwd_raw(q, one, one, one, 0, one, one, one, 0, 0,
-                                      B, 2, S, D, Tq, 4, QB, KB, S, dtype, 0)
+                                      B, 2, S, D, Tq, 4, QB, KB, P, S, dtype, 0)
     assert call(q=0) == 1
     assert call(B=0) == 2
     assert call(Tq=5) == 2            # Tq != ceil(S / QB)
+    assert call(P=-1) == 2            # negative number of stored partial tiles
     assert call(D=96) == 3
     assert call(D=256) == 3
     assert call(QB=32) == 4
@@ -57,7 +58,7 @@ def test_python_module_surface():
                  "omni_attn_preftech_kernel", "omni_attn_preftech",
                  "omni_attn_mma_stages_split_q_shared_kv_swizzle", "omni_attn_forward"):
         assert callable(getattr(omni_attn, name)), name
-    assert omni_attn.abi_version() == 1
+    assert omni_attn.abi_version() == 2
     assert os.path.dirname(omni_attn.__file__) == PKG
 
 
@@ -91,3 +92,34 @@ def test_wrappers_validate_before_launch():
                                  torch.zeros(1, 2, 256, 48, dtype=torch.float16), mask)
     with pytest.raises(ValueError, match="dtype"):
         omni_attention_shared_kv(q.float(), q.float(), q.float(), mask)
+
+
+def test_kernel_resources_of_the_built_library():
+    """The build records registers / scratch / occupancy of every kernel instance and refuses
+    instances that spill or lose occupancy; the record of the library in the tree passes the
+    same check (and the check itself rejects a spilling or low-occupancy record)."""
+    import importlib.util
+    import json
+    spec = importlib.util.spec_from_file_location("_omni_build", os.path.join(PKG, "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    if not os.path.exists(build.RESOURCES_JSON):
+        build.build_capi(jobs=4)
+    with open(build.RESOURCES_JSON) as f:
+        kernels = json.load(f)
+    fwd = {k: v for k, v in kernels.items() if "fwd_kernel" in k}
+    assert len(fwd) == 24
+    build.check_resources(kernels)
+    for name, r in fwd.items():
+        assert r["scratch_bytes"] == 0 and r["vgprs"] <= 256 and r["waves_per_simd"] >= 2, (name, r)
+    bad = {"k_fwd_kernel_x": {"scratch_bytes": 16, "vgpr_spills": 4, "sgpr_spills": 0, "waves_per_simd": 2}}
+    with pytest.raises(RuntimeError, match="scratch"):
+        build.check_resources(bad)
+    low = {"k_fwd_kernel_x": {"scratch_bytes": 0, "vgpr_spills": 0, "sgpr_spills": 0, "waves_per_simd": 1}}
+    with pytest.raises(RuntimeError, match="waves per SIMD"):
+        build.check_resources(low)
+    remarks = ("a.hpp:1:1: remark: Function Name: kern_a [-Rpass-analysis=kernel-resource-usage]\n"
+               "a.hpp:1:1: remark:     VGPRs: 77 [-Rpass-analysis=kernel-resource-usage]\n"
+               "a.hpp:1:1: remark:     ScratchSize [bytes/lane]: 8 [-Rpass-analysis=kernel-resource-usage]\n"
+               "a.hpp:1:1: remark:     Occupancy [waves/SIMD]: 5 [-Rpass-analysis=kernel-resource-usage]\n")
+    assert build.parse_resource_remarks(remarks) == {"kern_a": {"vgprs": 77, "scratch_bytes": 8, "waves_per_simd": 5}}

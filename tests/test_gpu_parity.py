@@ -90,21 +90,36 @@ def _merge_property(w, o, lse, device):
     assert (o_merged - o.float()).abs().max().item() <= 2 * TOL_O[w.dtype]
 
 
+def _oracle_slabs(name, B, H):
+    """(batch, head) slabs checked against the dense oracle.  The headline configurations
+    (c2, its 8K variant, c3) are checked on every slab; the two largest ones on at least 8
+    slabs that cover every distinct batch layout (heads of a batch element share their mask,
+    so the slabs of one batch element differ in q/k/v only)."""
+    if name in ("c2_interleaved", "c2_interleaved_8k", "c3_partial"):
+        return [(b, h) for b in range(B) for h in range(H)]
+    if name == "c4_long":
+        return [(0, h) for h in range(0, H, 4)]                  # 8 of 32 heads, one layout
+    if name == "c5_batched":
+        return [(b, (5 * b + 1) % H) for b in range(B)]           # all 8 layouts, different heads
+    return [(b, (3 * b) % H) for b in range(B)]                   # c5_full_control: 8 slabs
+
+
 @pytest.mark.parametrize("name", ["c2_interleaved", "c2_interleaved_8k", "c3_partial", "c4_long",
                                   "c5_batched", "c5_full_control"])
 def test_config_full_size(name, gpu_device):
-    """Full-size run; oracle on sampled (batch, head) slabs; merge property on all heads."""
+    """Full-size run against the dense oracle (slabs: see _oracle_slabs), plus the merge
+    property on all heads."""
     w = make_workload(name, seed=0)
     B, H, S, D = w.q.shape
     o, lse = run_workload(w, gpu_device)
     assert not torch.isnan(o).any() and not torch.isnan(lse).any()
-    samples = sorted({(0, 0), (B - 1, H - 1), (B // 2, H // 2)})
-    if name.startswith("c5"):
-        samples = sorted({(0, 0), (1, 1), (2, H - 1)}) if name == "c5_batched" else [(B - 1, 3)]
-    for b, h in samples:
-        mask = prefix_mask(w.prefix_len[b], S)
-        ro, rl = attention_dense_fp32(w.q[b, h], w.k[b, h], w.v[b, h], mask)
-        compare_with_oracle(o[b, h], lse[b, h], ro, rl, w.dtype, f"{name} slab ({b},{h})")
+    o_cpu, lse_cpu = o.cpu(), lse.cpu()
+    masks = {}
+    for b, h in _oracle_slabs(name, B, H):
+        if b not in masks:
+            masks = {b: prefix_mask(w.prefix_len[b], S)}
+        ro, rl = attention_dense_fp32(w.q[b, h], w.k[b, h], w.v[b, h], masks[b])
+        compare_with_oracle(o_cpu[b, h], lse_cpu[b, h], ro, rl, w.dtype, f"{name} slab ({b},{h})")
     _merge_property(w, o, lse, gpu_device)
 
 
@@ -164,6 +179,61 @@ def test_out_of_range_metadata_is_clamped(gpu_device):
     assert torch.equal(o, o2) and torch.equal(lse, lse2)
 
 
+def test_partial_index_beyond_the_stored_tiles_skips_the_slot(gpu_device):
+    """A PARTIAL slot whose index is >= the number of stored tiles has no bits: it is
+    skipped like a negative index, and nothing beyond the tile array is read.  Tiles are
+    laid out so that memory right behind the array is another, all-ones tensor: a kernel
+    that read tile P would attend everything and differ from the expected result."""
+    gen = torch.Generator().manual_seed(21)
+    S, D, QB, KB = 512, 64, 128, 128
+    q, k, v = (torch.randn(1, 2, S, D, generator=gen).to(torch.bfloat16) for _ in range(3))
+    Tq = Tk = S // QB
+    nb = torch.full((1, 2, Tq), Tk, dtype=torch.int32)
+    idx = torch.arange(Tk, dtype=torch.int32).expand(1, 2, Tq, Tk).contiguous()
+    tys = torch.full((1, 2, Tq, Tk), 3, dtype=torch.int32)
+    tys[..., 0] = 2  # one FULL slot per row so that no row is empty
+    P = 3
+    tiles = torch.rand(P, QB, KB, generator=gen) < 0.5
+    pidx = torch.randint(0, P, (1, 2, Tq, Tk), generator=gen, dtype=torch.int32)
+    bad = pidx.clone()
+    bad[0, 0, 1, 2] = P            # first index past the end
+    bad[0, 1, 2, 1] = 1 << 20      # far past the end
+    bad[0, 1, 3, 3] = 2 ** 31 - 1
+    skip = pidx.clone()
+    for pos in ((0, 0, 1, 2), (0, 1, 2, 1), (0, 1, 3, 3)):
+        skip[pos] = -1
+    backing = torch.ones(P + 4, QB, KB, dtype=torch.bool)  # tile P and beyond: all ones
+    backing[:P] = tiles
+    backing_d = backing.to(gpu_device)
+    o_bad, lse_bad = run_kernel(q, k, v, nb, idx, tys, QB, KB, S, bad, backing_d[:P], device=gpu_device)
+    o_skip, lse_skip = run_kernel(q, k, v, nb, idx, tys, QB, KB, S, skip, backing_d[:P], device=gpu_device)
+    assert torch.equal(o_bad, o_skip) and torch.equal(lse_bad, lse_skip)
+    wo, wl = attention_block_walk(q, k, v, nb, idx, tys, QB, KB, S, bad, tiles)
+    compare_with_oracle(o_bad, lse_bad, wo, wl, torch.bfloat16, "out-of-range partial index")
+
+
+def test_any_non_zero_mask_byte_means_attend(gpu_device):
+    """partial_block_masks is read as bytes: the reference's kernels test `!mask[...]`
+    (attn_naive.cu:151), so 2, 0x80 or 0xff attend like 1."""
+    gen = torch.Generator().manual_seed(22)
+    S, D, QB, KB = 256, 64, 128, 64
+    q, k, v = (torch.randn(1, 1, S, D, generator=gen).to(torch.float16) for _ in range(3))
+    Tq, Tk = S // QB, S // KB
+    nb = torch.full((1, 1, Tq), Tk, dtype=torch.int32)
+    idx = torch.arange(Tk, dtype=torch.int32).expand(1, 1, Tq, Tk).contiguous()
+    tys = torch.full((1, 1, Tq, Tk), 3, dtype=torch.int32)
+    pidx = torch.arange(Tq * Tk, dtype=torch.int32).view(1, 1, Tq, Tk)
+    bits = torch.rand(Tq * Tk, QB, KB, generator=gen) < 0.6
+    values = torch.tensor([1, 2, 4, 0x10, 0x80, 0xfe, 0xff, 3], dtype=torch.uint8)
+    pick = torch.randint(0, len(values), bits.shape, generator=gen)
+    as_bytes = torch.where(bits, values[pick], torch.zeros((), dtype=torch.uint8))
+    o1, l1 = run_kernel(q, k, v, nb, idx, tys, QB, KB, S, pidx, bits, device=gpu_device)
+    o2, l2 = run_kernel(q, k, v, nb, idx, tys, QB, KB, S, pidx, as_bytes, device=gpu_device)
+    assert torch.equal(o1, o2) and torch.equal(l1, l2)
+    wo, wl = attention_block_walk(q, k, v, nb, idx, tys, QB, KB, S, pidx, as_bytes)
+    compare_with_oracle(o2, l2, wo, wl, torch.float16, "non-zero mask bytes")
+
+
 def test_non_default_stream(gpu_device):
     w = make_workload("c1_causal", seed=2)
     o_ref, lse_ref = run_workload(w, gpu_device)
@@ -202,7 +272,7 @@ def test_runtime_is_linear_in_listed_blocks(gpu_device):
     width 1, 2, 4 ... 32 blocks): a straight line, t = a + b * N_ne."""
     import bench
 
-    r = bench.band_sweep(torch.device(gpu_device), steps=12, warmup=3)
+    r = bench.band_sweep(torch.device(gpu_device), steps=30, warmup=10)
     assert r["fit"]["r2"] > 0.98, r
     assert r["fit"]["ns_per_block"] > 0
 

@@ -113,6 +113,31 @@ def test_transfusion_rule_prefix_form_matches_bruteforce():
         assert torch.equal(prefix_mask(modality_prefix_lengths(mp, S), S)[0], brute), spans
 
 
+def test_transfusion_rule_known_answer_8x8():
+    """One image span (offset 2, length 3) in 8 tokens, written out by hand from the rule
+    allow[i, j] = (i >= j) or (i >= offset and j < offset + length)
+    (transfusion_pytorch/transfusion.py:496-515): tokens before the image are causal, tokens
+    of the image see the whole image, later tokens see the image through causality anyway.
+    Pins the brute-force restatement and the product's two forms by something that is neither."""
+    from omni_attn_torch import modality_prefix_lengths, naive_attn_mask
+    expected = torch.tensor([
+        [1, 0, 0, 0, 0, 0, 0, 0],
+        [1, 1, 0, 0, 0, 0, 0, 0],
+        [1, 1, 1, 1, 1, 0, 0, 0],
+        [1, 1, 1, 1, 1, 0, 0, 0],
+        [1, 1, 1, 1, 1, 0, 0, 0],
+        [1, 1, 1, 1, 1, 1, 0, 0],
+        [1, 1, 1, 1, 1, 1, 1, 0],
+        [1, 1, 1, 1, 1, 1, 1, 1]], dtype=torch.bool)
+    assert torch.equal(transfusion_mask_bruteforce(8, [(2, 3)]), expected)
+    mp = torch.tensor([[[1, 2, 3]]], dtype=torch.long)
+    assert torch.equal(naive_attn_mask(8, mp)[0], expected)
+    assert torch.equal(prefix_mask(modality_prefix_lengths(mp, 8), 8)[0], expected)
+    # a transposed or sign-flipped rule would give one of these instead
+    assert not torch.equal(expected, expected.t())
+    assert modality_prefix_lengths(mp, 8)[0].tolist() == [1, 2, 5, 5, 5, 6, 7, 8]
+
+
 @pytest.mark.parametrize("pat", load_printed_masks()["typed_block_patterns"], ids=lambda p: p["source"])
 def test_block_semantics_against_printed_sparsity(pat):
     """Typed block patterns + the sparsity the reference printed for their dense mask.
@@ -151,6 +176,38 @@ def test_block_walk_matches_dense_oracle(QB, KB):
         assert torch.allclose(lse[live], rl[live], atol=2e-5)
         assert (o[~live] == 0).all()
         assert (~live).any(), "the case must contain empty rows"
+
+
+def test_partial_index_beyond_the_stored_tiles_is_skipped_by_the_walk():
+    """An index >= the number of stored tiles means "no bits stored" (the product's contract;
+    the reference reads such an index unchecked, attn_naive.cu:124-131)."""
+    gen = torch.Generator().manual_seed(6)
+    q, k, v = (_rand(gen, 1, 1, 256, 32) for _ in range(3))
+    nb = torch.tensor([[[2, 2]]], dtype=torch.int32)
+    idx = torch.tensor([[[[0, 1], [0, 1]]]], dtype=torch.int32)
+    tys = torch.tensor([[[[2, 3], [3, 2]]]], dtype=torch.int32)
+    tiles = torch.rand(2, 128, 128, generator=gen) < 0.5
+    pidx_bad = torch.tensor([[[[-1, 2], [1 << 20, -1]]]], dtype=torch.int32)
+    pidx_none = torch.full((1, 1, 2, 2), -1, dtype=torch.int32)
+    a = attention_block_walk(q, k, v, nb, idx, tys, 128, 128, 256, pidx_bad, tiles)
+    b = attention_block_walk(q, k, v, nb, idx, tys, 128, 128, 256, pidx_none, tiles)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    pidx_ok = torch.tensor([[[[-1, 1], [0, -1]]]], dtype=torch.int32)
+    c = attention_block_walk(q, k, v, nb, idx, tys, 128, 128, 256, pidx_ok, tiles)
+    assert not torch.equal(a[0], c[0])
+
+
+def test_walk_treats_any_non_zero_mask_byte_as_attend():
+    gen = torch.Generator().manual_seed(7)
+    q, k, v = (_rand(gen, 1, 1, 128, 32) for _ in range(3))
+    nb = torch.tensor([[[1]]], dtype=torch.int32)
+    idx = torch.zeros(1, 1, 1, 1, dtype=torch.int32)
+    tys = torch.full((1, 1, 1, 1), 3, dtype=torch.int32)
+    pidx = torch.zeros(1, 1, 1, 1, dtype=torch.int32)
+    bits = torch.rand(1, 128, 128, generator=gen) < 0.5
+    a = attention_block_walk(q, k, v, nb, idx, tys, 128, 128, 128, pidx, bits)
+    b = attention_block_walk(q, k, v, nb, idx, tys, 128, 128, 128, pidx, bits.to(torch.uint8) * 0xfe)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
 
 
 def test_bitless_partial_slot_is_skipped_by_the_walk():
