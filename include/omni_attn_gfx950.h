@@ -107,6 +107,33 @@ int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v, void* o,
                          int seqlen_orig, int dtype, void* stream);
 
 /*
+ * Pre-pass for masks that are reused over many launches: packs the bool tiles that the
+ * reference's build_partial_block_data produces (omni-attn-mma/omni_attn_torch.py:148-205,
+ * [P, QB, KB] bytes) into [P, QB, KB / 32] 32-bit words, bit j of word c of a row = key
+ * 32 c + j of that row, any non-zero byte counting as set.  QB, KB in {64, 128};
+ * partial_masks 16-byte aligned.  Asynchronous on `stream`; allocates nothing.
+ */
+int omni_attn_pack_partial_masks_gfx950(const uint8_t* partial_masks, uint32_t* partial_bits,
+                                        int num_partial, int QB, int KB, void* stream);
+
+/*
+ * omni_attn_fwd_gfx950 with the PARTIAL tiles already packed by
+ * omni_attn_pack_partial_masks_gfx950 (same semantics and results bit for bit; the byte
+ * tiles of the reference's signature, omni-attn-mma/pybind/omni_attn.cc:10-68, are
+ * replaced by their packed form).
+ */
+int omni_attn_fwd_packed_gfx950(const void* q, const void* k, const void* v, void* o,
+                                float* lse_or_null,
+                                const int32_t* kv_num_blocks,
+                                const int32_t* kv_indices,
+                                const int32_t* block_mask_types,
+                                const int32_t* partial_idx_or_null,
+                                const uint32_t* partial_bits_or_null,
+                                int B, int H, int S_pad, int D,
+                                int Tq, int max_blocks, int QB, int KB, int num_partial,
+                                int seqlen_orig, int dtype, void* stream);
+
+/*
  * Measurement aid (no counterpart in the reference): enqueue a kernel that issues nothing but
  * 32x32x16 matrix instructions of `dtype` from registers -- two workgroups of four waves per
  * compute unit, `iters` x 8 instructions per wave -- so that a caller timing the launch can

@@ -122,7 +122,7 @@ def build_capi(jobs):
         cmds.append([HIPCC] + DEVICE_FLAGS + [
             "-DOMNI_INST_BF16=%d" % bf, "-DOMNI_INST_D=%d" % d,
             "-c", os.path.join(CSRC, "omni_attn_fwd_inst.hip"), "-o", obj])
-    for src in ("omni_attn_capi", "omni_attn_probe"):
+    for src in ("omni_attn_capi", "omni_attn_probe", "omni_attn_mask_pack"):
         obj = os.path.join(OBJ, src + ".o")
         objs.append(obj)
         cmds.append([HIPCC] + DEVICE_FLAGS + ["-c", os.path.join(CSRC, src + ".hip"), "-o", obj])

@@ -64,20 +64,21 @@ int query_topology(DeviceTopology* out) {
 }
 }  // namespace
 
-extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v, void* o,
-                                    float* lse_or_null, const int32_t* kv_num_blocks,
-                                    const int32_t* kv_indices, const int32_t* block_mask_types,
-                                    const int32_t* partial_idx_or_null,
-                                    const uint8_t* partial_masks_or_null, int B, int H, int S_pad,
-                                    int D, int Tq, int max_blocks, int QB, int KB, int num_partial,
-                                    int seqlen_orig, int dtype, void* stream) {
+namespace {
+// Both forward entry points: PARTIAL tiles as bytes (partial_masks) or packed (partial_bits).
+int forward(const void* q, const void* k, const void* v, void* o, float* lse_or_null,
+            const int32_t* kv_num_blocks, const int32_t* kv_indices, const int32_t* block_mask_types,
+            const int32_t* partial_idx_or_null, const uint8_t* partial_masks_or_null,
+            const uint32_t* partial_bits_or_null, int B, int H, int S_pad, int D, int Tq,
+            int max_blocks, int QB, int KB, int num_partial, int seqlen_orig, int dtype, void* stream) {
   using namespace omni_attn;
   if (!q || !k || !v || !o || !kv_num_blocks || !kv_indices || !block_mask_types)
     return OMNI_ATTN_ERR_NULL_POINTER;
   // 16-byte loads and stores on q, k, v, o and the mask tiles; 4-byte ones on the rest
   const auto misaligned = [](const void* ptr, uintptr_t a) { return (reinterpret_cast<uintptr_t>(ptr) & (a - 1)) != 0; };
   if (misaligned(q, 16) || misaligned(k, 16) || misaligned(v, 16) || misaligned(o, 16) ||
-      misaligned(partial_masks_or_null, 16) || misaligned(lse_or_null, 4) || misaligned(kv_num_blocks, 4) ||
+      misaligned(partial_masks_or_null, 16) || misaligned(partial_bits_or_null, 4) ||
+      misaligned(lse_or_null, 4) || misaligned(kv_num_blocks, 4) ||
       misaligned(kv_indices, 4) || misaligned(block_mask_types, 4) || misaligned(partial_idx_or_null, 4))
     return OMNI_ATTN_ERR_MISALIGNED;
   if (dtype != OMNI_ATTN_DTYPE_F16 && dtype != OMNI_ATTN_DTYPE_BF16)
@@ -102,9 +103,11 @@ extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v,
   p.kv_indices = kv_indices;
   p.types = block_mask_types;
   if ((long long)num_partial * QB * KB > 0x7fffffffLL * 64) return OMNI_ATTN_ERR_TOO_LARGE;
-  const bool has_partial = partial_idx_or_null != nullptr && partial_masks_or_null != nullptr && num_partial > 0;
+  const bool has_partial = partial_idx_or_null != nullptr && num_partial > 0 &&
+                           (partial_masks_or_null != nullptr || partial_bits_or_null != nullptr);
   p.partial_idx = has_partial ? partial_idx_or_null : nullptr;
   p.partial_masks = has_partial ? partial_masks_or_null : nullptr;
+  p.partial_bits = has_partial ? partial_bits_or_null : nullptr;
   p.num_partial = has_partial ? num_partial : 0;
   p.S = S_pad;
   p.Tq = Tq;
@@ -153,6 +156,31 @@ extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v,
     return OMNI_ATTN_ERR_LAUNCH;
   }
   return OMNI_ATTN_OK;
+}
+}  // namespace
+
+extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v, void* o,
+                                    float* lse_or_null, const int32_t* kv_num_blocks,
+                                    const int32_t* kv_indices, const int32_t* block_mask_types,
+                                    const int32_t* partial_idx_or_null,
+                                    const uint8_t* partial_masks_or_null, int B, int H, int S_pad,
+                                    int D, int Tq, int max_blocks, int QB, int KB, int num_partial,
+                                    int seqlen_orig, int dtype, void* stream) {
+  return forward(q, k, v, o, lse_or_null, kv_num_blocks, kv_indices, block_mask_types, partial_idx_or_null,
+                 partial_masks_or_null, nullptr, B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial,
+                 seqlen_orig, dtype, stream);
+}
+
+extern "C" int omni_attn_fwd_packed_gfx950(const void* q, const void* k, const void* v, void* o,
+                                           float* lse_or_null, const int32_t* kv_num_blocks,
+                                           const int32_t* kv_indices, const int32_t* block_mask_types,
+                                           const int32_t* partial_idx_or_null,
+                                           const uint32_t* partial_bits_or_null, int B, int H, int S_pad,
+                                           int D, int Tq, int max_blocks, int QB, int KB, int num_partial,
+                                           int seqlen_orig, int dtype, void* stream) {
+  return forward(q, k, v, o, lse_or_null, kv_num_blocks, kv_indices, block_mask_types, partial_idx_or_null,
+                 nullptr, partial_bits_or_null, B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial,
+                 seqlen_orig, dtype, stream);
 }
 
 extern "C" const char* omni_attn_status_string(int status) {

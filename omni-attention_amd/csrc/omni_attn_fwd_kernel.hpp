@@ -63,6 +63,8 @@ struct FwdParams {
   const int32_t* types;          // [B,H,Tq,max_blocks]
   const int32_t* partial_idx;    // [B,H,Tq,max_blocks] or null
   const uint8_t* partial_masks;  // [P,QB,KB] bytes or null
+  const uint32_t* partial_bits;  // [P,QB,KB/32] words (bit j of word c = key 32c + j) or null;
+                                 // at most one of partial_masks / partial_bits is set
   int num_partial; // P: tiles stored in partial_masks
   int S;           // padded sequence length (rows per (b,h) slab)
   int Tq;          // query blocks per slab
@@ -206,6 +208,24 @@ __device__ __forceinline__ void buffer_to_lds_b128(i32x4_t rsrc, uint32_t lane_o
         "s"(__builtin_amdgcn_readfirstlane(uniform_off))
       : "memory", "m0");
 }
+// 4 bytes per lane: the dword of lane l lands at lds_base + 4 * l (lanes switched off by the
+// execution mask neither load nor store).
+__device__ __forceinline__ void buffer_to_lds_b32(i32x4_t rsrc, uint32_t lane_off,
+                                                  uint32_t uniform_off, uint32_t lds_base) {
+  i32x4_t r;
+  r[0] = __builtin_amdgcn_readfirstlane(rsrc[0]);
+  r[1] = __builtin_amdgcn_readfirstlane(rsrc[1]);
+  r[2] = __builtin_amdgcn_readfirstlane(rsrc[2]);
+  r[3] = __builtin_amdgcn_readfirstlane(rsrc[3]);
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dword %1, %2, %3 offen lds"
+      :
+      : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(lane_off), "s"(r),
+        "s"(__builtin_amdgcn_readfirstlane(uniform_off))
+      : "memory", "m0");
+}
 // Block-mask metadata is read-only for the whole launch and every read of it is
 // wave-uniform: reading it through the constant address space makes these scalar loads
 // (SGPR results, no vector-memory latency in the instruction stream).
@@ -305,7 +325,8 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   // instruction per step.  A new chunk is fetched when the walk reaches it (every 64
   // blocks).  The loads of a chunk do not depend on the block count, so the first chunk,
   // the count and Q are all in flight together at the start of the kernel.
-  const bool has_partial = p.partial_idx != nullptr && p.partial_masks != nullptr;
+  const bool packed_tiles = p.partial_bits != nullptr;
+  const bool has_partial = p.partial_idx != nullptr && (p.partial_masks != nullptr || packed_tiles);
   int32_t mv_row0 = 0, mv_mode = kMasked, mv_pid = -1;
   auto load_chunk = [&](int chunk) {
     const int j = chunk * 64 + lane;
@@ -397,6 +418,19 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
       const uint32_t row = uint32_t(32 * w + i * (64 / MCPR)) + uint32_t(lane / MCPR);
       buffer_to_lds_b128(rM, row * uint32_t(KB) + uint32_t(lane % MCPR) * 16u, uint32_t(half * STEP),
                          dst + uint32_t(i) * 1024u);
+    }
+  };
+  // Tiles that arrive already packed (one 32-bit word per row and 32 keys) need no second
+  // stage: one 4-byte buffer->LDS load per lane puts the step's words of the wave's 32 rows
+  // where the byte path parks the words it packs.
+  auto prefetch_mask_words = [&](int it, const StepInfo& si) {
+    constexpr uint32_t TILE_WORDS = uint32_t(QB) * (KB / 32);
+    const int half = it % SPB;
+    const i32x4_t rM = make_buffer_resource(p.partial_bits + size_t(si.pid) * TILE_WORDS, TILE_WORDS * 4u);
+    if (lane < 32 * NTL) {
+      const uint32_t row = uint32_t(32 * w + lane / NTL);
+      buffer_to_lds_b32(rM, (row * uint32_t(KB / 32) + uint32_t(lane % NTL)) * 4u, uint32_t(half * NTL) * 4u,
+                        lds_offset_of(sBits) + uint32_t(32 * w * NTL) * 4u);
     }
   };
   auto stage_mask_bits = [&]() {
@@ -617,8 +651,12 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
       issue_load(NCH + i, 1, nxt.row0, 0);
     }
     if (cur.mode == kPartial) {
-      prefetch_mask_bytes(0, cur);
-      stage_mask_bits();
+      if (packed_tiles) {
+        prefetch_mask_words(0, cur);
+      } else {
+        prefetch_mask_bytes(0, cur);
+        stage_mask_bits();
+      }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
@@ -642,9 +680,15 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     }
     if (!unmasked(cur)) apply_mask(IntC<SET>{}, cur);
     const bool next_partial = it + 1 < nsteps && nxt.mode == kPartial;
-    if (next_partial) prefetch_mask_bytes(it + 1, nxt);
+    if (next_partial) {
+      if (packed_tiles) {
+        prefetch_mask_words(it + 1, nxt);
+      } else {
+        prefetch_mask_bytes(it + 1, nxt);
+      }
+    }
     body(IntC<SET>{}, first_c, nn.row0, cur.row0);
-    if (next_partial) stage_mask_bits();
+    if (next_partial && !packed_tiles) stage_mask_bits();
     const StepInfo n3 = step_info(it + 3);
     cur = nxt;
     nxt = nn;

@@ -41,7 +41,7 @@ void forward_impl(const torch::Tensor& Q, const torch::Tensor& K, const torch::T
                   const torch::Tensor& kv_indices, const torch::Tensor& block_mask_types,
                   int Q_BLOCK_SIZE, int KV_BLOCK_SIZE, int seqlen_orig,
                   const torch::Tensor& partial_block_mask_indices,
-                  const torch::Tensor& partial_block_masks, bool has_partial) {
+                  const torch::Tensor& partial_block_masks, bool has_partial, bool packed = false) {
   if (Q.scalar_type() != torch::kHalf && Q.scalar_type() != torch::kBFloat16)
     throw std::runtime_error("Tensor dtype mismatch: Q must be torch.float16 or torch.bfloat16");
   check_qkvo(Q, "Q", Q);
@@ -86,22 +86,25 @@ void forward_impl(const torch::Tensor& Q, const torch::Tensor& K, const torch::T
     if (partial_block_mask_indices.scalar_type() != torch::kInt32)
       throw std::runtime_error(
           "Tensor dtype mismatch: partial_block_mask_indices must be torch.int32");
-    if (partial_block_masks.scalar_type() != torch::kBool)
+    if (!packed && partial_block_masks.scalar_type() != torch::kBool)
       throw std::runtime_error("Tensor dtype mismatch: partial_block_masks must be torch.bool");
+    if (packed && partial_block_masks.scalar_type() != torch::kInt32)
+      throw std::runtime_error("Tensor dtype mismatch: packed partial tiles must be torch.int32");
     if (!partial_block_mask_indices.is_contiguous() || !partial_block_masks.is_contiguous())
       throw std::runtime_error("Partial block mask tensors must be contiguous.");
     if (partial_block_mask_indices.sizes() != kv_indices.sizes())
       throw std::runtime_error("partial_block_mask_indices must have the shape of kv_indices");
     if (partial_block_masks.dim() != 3 || partial_block_masks.size(1) != Q_BLOCK_SIZE ||
-        partial_block_masks.size(2) != KV_BLOCK_SIZE)
+        partial_block_masks.size(2) != (packed ? KV_BLOCK_SIZE / 32 : KV_BLOCK_SIZE))
       throw std::runtime_error(
-          "partial_block_masks must be [num_partial, Q_BLOCK_SIZE, KV_BLOCK_SIZE]");
+          packed ? "packed partial tiles must be [num_partial, Q_BLOCK_SIZE, KV_BLOCK_SIZE / 32]"
+                 : "partial_block_masks must be [num_partial, Q_BLOCK_SIZE, KV_BLOCK_SIZE]");
     if (partial_block_mask_indices.device() != Q.device() ||
         partial_block_masks.device() != Q.device())
       throw std::runtime_error("Partial block mask tensors must be on the device of Q");
     if (partial_block_masks.size(0) > 0) {
       pidx = partial_block_mask_indices.data_ptr<int32_t>();
-      pmask = reinterpret_cast<const uint8_t*>(partial_block_masks.data_ptr<bool>());
+      pmask = static_cast<const uint8_t*>(partial_block_masks.data_ptr());
       num_partial = int(partial_block_masks.size(0));
     }
   }
@@ -109,12 +112,19 @@ void forward_impl(const torch::Tensor& Q, const torch::Tensor& K, const torch::T
   c10::DeviceGuard guard(Q.device());
   hipStream_t stream = c10::hip::getCurrentHIPStream(Q.device().index()).stream();
   const int dtype = Q.scalar_type() == torch::kBFloat16 ? OMNI_ATTN_DTYPE_BF16 : OMNI_ATTN_DTYPE_F16;
-  const int rc = omni_attn_fwd_gfx950(
-      Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), lse,
-      kv_num_blocks.data_ptr<int32_t>(), kv_indices.data_ptr<int32_t>(),
-      block_mask_types.data_ptr<int32_t>(), pidx, pmask, int(B), int(H), int(S), int(D),
-      int(num_q_blocks), int(max_blocks), Q_BLOCK_SIZE, KV_BLOCK_SIZE, num_partial, seqlen_orig, dtype,
-      static_cast<void*>(stream));
+  const int rc =
+      packed ? omni_attn_fwd_packed_gfx950(
+                   Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), lse,
+                   kv_num_blocks.data_ptr<int32_t>(), kv_indices.data_ptr<int32_t>(),
+                   block_mask_types.data_ptr<int32_t>(), pidx, reinterpret_cast<const uint32_t*>(pmask),
+                   int(B), int(H), int(S), int(D), int(num_q_blocks), int(max_blocks), Q_BLOCK_SIZE,
+                   KV_BLOCK_SIZE, num_partial, seqlen_orig, dtype, static_cast<void*>(stream))
+             : omni_attn_fwd_gfx950(
+                   Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), lse,
+                   kv_num_blocks.data_ptr<int32_t>(), kv_indices.data_ptr<int32_t>(),
+                   block_mask_types.data_ptr<int32_t>(), pidx, pmask, int(B), int(H), int(S), int(D),
+                   int(num_q_blocks), int(max_blocks), Q_BLOCK_SIZE, KV_BLOCK_SIZE, num_partial,
+                   seqlen_orig, dtype, static_cast<void*>(stream));
   if (rc != OMNI_ATTN_OK) {
     std::string msg = std::string("omni_attn: ") + omni_attn_status_string(rc);
     if (rc == OMNI_ATTN_ERR_UNSUPPORTED_HEAD_DIM) msg += ", got head_dim=" + std::to_string(D);
@@ -154,6 +164,42 @@ void omni_attn_forward(torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch:
                partial_block_masks, has_partial);
 }
 
+// PARTIAL tiles [P, QB, KB] bool -> [P, QB, KB / 32] int32 words, packed on the GPU.
+torch::Tensor omni_attn_pack_partial_masks(torch::Tensor partial_block_masks) {
+  if (!partial_block_masks.is_cuda() || partial_block_masks.scalar_type() != torch::kBool ||
+      partial_block_masks.dim() != 3 || !partial_block_masks.is_contiguous())
+    throw std::runtime_error("partial_block_masks must be a contiguous [P, Q_BLOCK_SIZE, KV_BLOCK_SIZE] bool GPU tensor");
+  const int64_t P = partial_block_masks.size(0), QB = partial_block_masks.size(1), KB = partial_block_masks.size(2);
+  if (KB % 32 != 0) throw std::runtime_error("KV_BLOCK_SIZE must be a multiple of 32");
+  c10::DeviceGuard guard(partial_block_masks.device());
+  torch::Tensor out = torch::empty({P, QB, KB / 32}, partial_block_masks.options().dtype(torch::kInt32));
+  hipStream_t stream = c10::hip::getCurrentHIPStream(partial_block_masks.device().index()).stream();
+  const int rc = omni_attn_pack_partial_masks_gfx950(
+      static_cast<const uint8_t*>(partial_block_masks.data_ptr()),
+      reinterpret_cast<uint32_t*>(out.data_ptr<int32_t>()), int(P), int(QB), int(KB), static_cast<void*>(stream));
+  if (rc != OMNI_ATTN_OK) throw std::runtime_error(std::string("omni_attn: ") + omni_attn_status_string(rc));
+  return out;
+}
+
+// omni_attn_forward with packed PARTIAL tiles; LSE may be an empty tensor (no logsumexp).
+void omni_attn_forward_packed(torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch::Tensor O,
+                              torch::Tensor LSE, torch::Tensor kv_num_blocks, torch::Tensor kv_indices,
+                              torch::Tensor block_mask_types, int Q_BLOCK_SIZE, int KV_BLOCK_SIZE,
+                              int seqlen_orig, torch::Tensor partial_block_mask_indices,
+                              torch::Tensor partial_block_bits) {
+  float* lse = nullptr;
+  if (LSE.numel() > 0) {
+    if (LSE.scalar_type() != torch::kFloat32)
+      throw std::runtime_error("Tensor dtype mismatch: LSE must be torch.float32");
+    if (!LSE.is_contiguous() || LSE.dim() != 3 || Q.dim() != 4 || LSE.size(0) != Q.size(0) ||
+        LSE.size(1) != Q.size(1) || LSE.size(2) != Q.size(2) || LSE.device() != Q.device())
+      throw std::runtime_error("LSE must be a contiguous [B, H, S] tensor on the device of Q");
+    lse = LSE.data_ptr<float>();
+  }
+  forward_impl(Q, K, V, O, lse, kv_num_blocks, kv_indices, block_mask_types, Q_BLOCK_SIZE, KV_BLOCK_SIZE,
+               seqlen_orig, partial_block_mask_indices, partial_block_bits, true, true);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -167,5 +213,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("omni_attn_mma_stages_split_q_shared_kv_swizzle", &omni_attn_op,
         "omni_attn_mma_stages_split_q_shared_kv_swizzle");
   m.def("omni_attn_forward", &omni_attn_forward, "omni_attn_forward (also writes logsumexp)");
+  m.def("omni_attn_pack_partial_masks", &omni_attn_pack_partial_masks,
+        "omni_attn_pack_partial_masks (bool tiles -> 32-bit words)");
+  m.def("omni_attn_forward_packed", &omni_attn_forward_packed,
+        "omni_attn_forward_packed (PARTIAL tiles as packed words)");
   m.def("abi_version", []() { return omni_attn_abi_version(); });
 }

@@ -19,6 +19,8 @@ DTYPE_BF16 = 1
 
 EXPORTED_SYMBOLS = (
     "omni_attn_fwd_gfx950",
+    "omni_attn_fwd_packed_gfx950",
+    "omni_attn_pack_partial_masks_gfx950",
     "omni_attn_mfma_peak_probe_gfx950",
     "omni_attn_status_string",
     "omni_attn_last_hip_error",
@@ -35,6 +37,10 @@ def load_library() -> ctypes.CDLL:
         vp, i32 = ctypes.c_void_p, ctypes.c_int
         lib.omni_attn_fwd_gfx950.restype = i32
         lib.omni_attn_fwd_gfx950.argtypes = [vp] * 10 + [i32] * 11 + [vp]
+        lib.omni_attn_fwd_packed_gfx950.restype = i32
+        lib.omni_attn_fwd_packed_gfx950.argtypes = [vp] * 10 + [i32] * 11 + [vp]
+        lib.omni_attn_pack_partial_masks_gfx950.restype = i32
+        lib.omni_attn_pack_partial_masks_gfx950.argtypes = [vp, vp, i32, i32, i32, vp]
         lib.omni_attn_mfma_peak_probe_gfx950.restype = i32
         lib.omni_attn_mfma_peak_probe_gfx950.argtypes = [i32, i32, vp, ctypes.POINTER(ctypes.c_double), vp]
         lib.omni_attn_status_string.restype = ctypes.c_char_p
@@ -73,11 +79,30 @@ def fwd_raw(q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, nb_ptr, idx_ptr, types_ptr, pid
         B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial, seqlen_orig, dtype, stream_ptr)
 
 
+def pack_partial_masks(partial_masks: torch.Tensor, stream: Optional[int] = None) -> torch.Tensor:
+    """[P, QB, KB] bool / uint8 tiles on the GPU -> [P, QB, KB // 32] int32 words (the bit
+    pattern of the library's uint32 words), packed by the library's pre-pass kernel."""
+    if not (partial_masks.is_cuda and partial_masks.is_contiguous() and partial_masks.dim() == 3
+            and partial_masks.dtype in (torch.bool, torch.uint8)):
+        raise RuntimeError("partial_masks must be a contiguous [P, QB, KB] bool GPU tensor")
+    P, QB, KB = partial_masks.shape
+    out = torch.empty(P, QB, KB // 32, dtype=torch.int32, device=partial_masks.device)
+    if stream is None:
+        stream = torch.cuda.current_stream(partial_masks.device).cuda_stream
+    with torch.cuda.device(partial_masks.device):
+        rc = load_library().omni_attn_pack_partial_masks_gfx950(partial_masks.data_ptr(), out.data_ptr(), P, QB, KB, stream)
+    if rc != 0:
+        raise RuntimeError("omni_attn_pack_partial_masks_gfx950: %s (status %d)" % (status_string(rc), rc))
+    return out
+
+
 def fwd(q, k, v, o, lse, kv_num_blocks, kv_indices, block_mask_types, QB, KB, seqlen_orig,
-        partial_idx=None, partial_masks=None, stream: Optional[int] = None) -> None:
+        partial_idx=None, partial_masks=None, stream: Optional[int] = None, partial_bits=None) -> None:
     """Enqueue the forward on ``stream`` (default: torch's current stream of q's device).
     q, k, v, o: contiguous [B, H, S_pad, D] fp16 or bf16 on the GPU; lse: fp32 [B, H, S_pad]
-    or None.  Raises RuntimeError with the library's message on a non-zero status."""
+    or None.  PARTIAL tiles either as bytes (``partial_masks``) or packed by
+    ``pack_partial_masks`` (``partial_bits``).  Raises RuntimeError with the library's message
+    on a non-zero status."""
     B, H, S, D = q.shape
     for t in (q, k, v, o):
         if not (t.is_cuda and t.is_contiguous() and t.dtype == q.dtype and t.shape == q.shape):
@@ -99,6 +124,21 @@ def fwd(q, k, v, o, lse, kv_num_blocks, kv_indices, block_mask_types, QB, KB, se
             partial_idx, partial_masks = None, None
     if stream is None:
         stream = torch.cuda.current_stream(q.device).cuda_stream
+    if partial_bits is not None:
+        if partial_masks is not None:
+            raise RuntimeError("pass partial_masks or partial_bits, not both")
+        if not (partial_bits.is_cuda and partial_bits.is_contiguous() and partial_bits.dtype == torch.int32
+                and partial_bits.dim() == 3 and partial_bits.shape[1:] == (QB, KB // 32)):
+            raise RuntimeError("partial_bits must be a contiguous [P, QB, KB // 32] int32 GPU tensor")
+        with torch.cuda.device(q.device):
+            rc = load_library().omni_attn_fwd_packed_gfx950(
+                _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(kv_num_blocks), _ptr(kv_indices),
+                _ptr(block_mask_types), _ptr(partial_idx if partial_bits.shape[0] else None),
+                _ptr(partial_bits if partial_bits.shape[0] else None), B, H, S, D, kv_num_blocks.shape[2],
+                kv_indices.shape[3], QB, KB, int(partial_bits.shape[0]), int(seqlen_orig), dtype, stream)
+        if rc != 0:
+            raise RuntimeError("omni_attn_fwd_packed_gfx950: %s (status %d)" % (status_string(rc), rc))
+        return
     with torch.cuda.device(q.device):
         rc = fwd_raw(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(kv_num_blocks),
                      _ptr(kv_indices), _ptr(block_mask_types), _ptr(partial_idx), _ptr(partial_masks),

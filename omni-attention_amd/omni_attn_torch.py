@@ -52,6 +52,9 @@ class OmniBlockMask:
     q_len, kv_len    padded lengths (multiples of the block sizes)
     partial_block_mask_indices  [B, H, num_q_blocks, max_blocks] int32, -1 = none
     partial_block_masks         [P, Q_BLOCK_SIZE, KV_BLOCK_SIZE] bool
+    partial_block_bits          [P, Q_BLOCK_SIZE, KV_BLOCK_SIZE // 32] int32: the same tiles, one
+                                bit per element, filled by pack_partial_masks() (not in the
+                                reference; the wrappers use it when it is there)
     """
     kv_num_blocks: Tensor
     kv_indices: Tensor
@@ -62,6 +65,17 @@ class OmniBlockMask:
     KV_BLOCK_SIZE: int = 128
     partial_block_mask_indices: Optional[Tensor] = None
     partial_block_masks: Optional[Tensor] = None
+    partial_block_bits: Optional[Tensor] = None
+
+    def pack_partial_masks(self) -> "OmniBlockMask":
+        """Pack the PARTIAL tiles once (on the GPU, by the extension's pre-pass kernel) for a mask
+        that is used for many launches; the wrappers then pass the packed words."""
+        if self.partial_block_masks is not None and self.partial_block_masks.numel() > 0:
+            if not self.partial_block_masks.is_cuda:
+                raise ValueError("pack_partial_masks needs the mask on the GPU: mask.to(device) first")
+            self.partial_block_bits = _load_extension().omni_attn_pack_partial_masks(
+                self.partial_block_masks.to(torch.bool).contiguous())
+        return self
 
     @property
     def num_q_blocks(self) -> int:
@@ -85,7 +99,7 @@ class OmniBlockMask:
         return OmniBlockMask(
             mv(self.kv_num_blocks), mv(self.kv_indices), mv(self.block_mask_types),
             self.q_len, self.kv_len, self.Q_BLOCK_SIZE, self.KV_BLOCK_SIZE,
-            mv(self.partial_block_mask_indices), mv(self.partial_block_masks))
+            mv(self.partial_block_mask_indices), mv(self.partial_block_masks), mv(self.partial_block_bits))
 
     def to_dense_mask(self, partial_fallback: str = "causal") -> Tensor:
         """Dense bool mask [B, H, q_len, kv_len], True = attend.
@@ -535,6 +549,16 @@ def _omni_attention(op_name: str, query: Tensor, key: Tensor, value: Tensor,
         partial_idx = torch.empty(0, dtype=torch.int32, device=dev)
         partial_masks = torch.empty(0, dtype=torch.bool, device=dev)
 
+    if has_partial and block_mask.partial_block_bits is not None and block_mask.partial_block_bits.device == dev:
+        # tiles packed once by OmniBlockMask.pack_partial_masks(): same kernel, packed input
+        lse_padded = (torch.empty(B, H, S_pad, dtype=torch.float32, device=dev) if return_lse
+                      else torch.empty(0, dtype=torch.float32, device=dev))
+        ext.omni_attn_forward_packed(query_padded, key_padded, value_padded, output_padded, lse_padded,
+                                     kv_num_blocks, kv_indices, block_mask_types, QB, KB, q_orig_len,
+                                     partial_idx, block_mask.partial_block_bits.contiguous())
+        if return_lse:
+            return output_padded[:, :, :q_orig_len, :], lse_padded[:, :, :q_orig_len]
+        return output_padded[:, :, :q_orig_len, :]
     if return_lse:
         lse_padded = torch.empty(B, H, S_pad, dtype=torch.float32, device=dev)
         ext.omni_attn_forward(query_padded, key_padded, value_padded, output_padded, lse_padded,
