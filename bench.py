@@ -259,6 +259,9 @@ def main(argv=None):
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the measured MFMA peak and the c2_interleaved_8k figure")
     ap.add_argument("--kernel-source-hash", action="store_true", help="print the hash and exit")
+    ap.add_argument("--backward", action="store_true",
+                    help="time the backward (dQ kernel + dK/dV kernel) instead of the forward; effective "
+                         "flops are 10*QB*KB*D per listed block (five products)")
     ap.add_argument("--packed-tiles", action="store_true",
                     help="pack the PARTIAL tiles once with the pre-pass kernel and time the forward on "
                          "packed tiles; also reports the pre-pass kernel against the HBM roofline")
@@ -328,8 +331,24 @@ def main(argv=None):
                        "us_per_launch": us, "tiles": int(pm.shape[0]),
                        "note": "launch plus allocation of the output by the caller's allocator included"}
 
+    bwd_state = None
+    if args.backward:
+        g = torch.Generator(device="cpu").manual_seed(args.seed + 1)
+        dout = torch.randn(w.q.shape, generator=g).to(w.dtype).to(dev)
+        omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, pidx,
+                           None if bits is not None else pm, stream=stream.cuda_stream, partial_bits=bits)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+        ws = torch.empty(omni_attn_capi.load_library().omni_attn_bwd_workspace_bytes(B, H, S), dtype=torch.uint8,
+                         device=dev)
+        bwd_state = (dout, dq, dk, dv, ws)
+
     def step():
-        if bits is not None:
+        if bwd_state is not None:
+            dout, dq, dk, dv, ws = bwd_state
+            omni_attn_capi.bwd(q, k, v, o, dout, lse, dq, dk, dv, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE,
+                               S, pidx, None if bits is not None else pm, bits, workspace=ws,
+                               stream=stream.cuda_stream)
+        elif bits is not None:
             omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, pidx, None,
                                stream=stream.cuda_stream, partial_bits=bits)
         else:
@@ -373,7 +392,7 @@ def main(argv=None):
     avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
     med_kernel_ms = statistics.median(kernel_ms)
     ms_per_step = wall / args.steps * 1e3
-    flops = w.effective_flops
+    flops = w.effective_flops * (2.5 if args.backward else 1.0)
     value = flops / (ms_per_step * 1e-3) / 1e12
     achieved = flops / (avg_kernel_ms * 1e-3) / 1e12
     traffic, traffic_provenance = traffic_for(args.workload)
@@ -413,6 +432,8 @@ def main(argv=None):
             "kernel_ms_avg": avg_kernel_ms,
         },
     }
+    if args.backward:
+        out["config"]["pass"] = "backward (dQ kernel + dK/dV kernel), 10*QB*KB*D flop per listed block"
     if pack_report is not None:
         out["mask_pack"] = pack_report
         out["config"]["partial_tiles"] = "packed once by the pre-pass kernel"

@@ -48,8 +48,9 @@ enum omni_attn_status {
   OMNI_ATTN_ERR_UNSUPPORTED_DTYPE = 5,
   OMNI_ATTN_ERR_LAUNCH = 6,            /* hipLaunch failed; see omni_attn_last_hip_error() */
   OMNI_ATTN_ERR_TOO_LARGE = 7,         /* a tensor exceeds 2^31-1 elements per (b,h) slab */
-  OMNI_ATTN_ERR_MISALIGNED = 8         /* q, k, v, o or partial masks not 16-byte aligned, or a
+  OMNI_ATTN_ERR_MISALIGNED = 8,        /* q, k, v, o or partial masks not 16-byte aligned, or a
                                           32-bit array not 4-byte aligned */
+  OMNI_ATTN_ERR_WORKSPACE = 9          /* workspace smaller than omni_attn_bwd_workspace_bytes() */
 };
 
 /*
@@ -132,6 +133,41 @@ int omni_attn_fwd_packed_gfx950(const void* q, const void* k, const void* v, voi
                                 int B, int H, int S_pad, int D,
                                 int Tq, int max_blocks, int QB, int KB, int num_partial,
                                 int seqlen_orig, int dtype, void* stream);
+
+/*
+ * Backward of omni_attn_fwd_gfx950: gradients of a scalar loss with respect to q, k and v,
+ * given dout = dLoss/dO and the o and lse the forward wrote for the same q, k, v and mask.
+ * The reference's operator is forward-only (omni-attn-mma/pybind/omni_attn.cc:70-77 exports no
+ * backward); this is what a caller needs to put the operator into the attention layer of
+ * transfusion_pytorch/transfusion.py:953-983 for training.  What is differentiated is exactly
+ * the forward's function: listed blocks only, FULL / CAUSAL / PARTIAL / MASKED semantics,
+ * scale 1/sqrt(D), rows >= seqlen_orig and rows with no allowed key get zero gradients.
+ *
+ *   dout, dq, dk, dv  [B, H, S_pad, D], same 16-bit type as q.  dq, dk, dv are written
+ *                     completely (rows of K/V that no query attends get zeros).
+ *   lse               [B, H, S_pad] fp32 as written by the forward (required).
+ *   partial tiles     as bytes (partial_masks_or_null) or packed (partial_bits_or_null);
+ *                     pass one of them or neither.
+ *   workspace         device memory of at least omni_attn_bwd_workspace_bytes(B, H, S_pad)
+ *                     bytes, 4-byte aligned; holds rowsum(dout . o) between the two kernels
+ *                     of the backward.  Contents before and after the call are meaningless.
+ * Limits beyond the forward's: Tq * ceil(max_blocks / 64) <= 4096 (OMNI_ATTN_ERR_TOO_LARGE).
+ * Two kernels are enqueued on `stream`; nothing is allocated; results are bitwise reproducible.
+ */
+size_t omni_attn_bwd_workspace_bytes(int B, int H, int S_pad);
+int omni_attn_bwd_gfx950(const void* q, const void* k, const void* v, const void* o,
+                         const void* dout, const float* lse,
+                         void* dq, void* dk, void* dv,
+                         const int32_t* kv_num_blocks,
+                         const int32_t* kv_indices,
+                         const int32_t* block_mask_types,
+                         const int32_t* partial_idx_or_null,
+                         const uint8_t* partial_masks_or_null,
+                         const uint32_t* partial_bits_or_null,
+                         void* workspace, size_t workspace_bytes,
+                         int B, int H, int S_pad, int D,
+                         int Tq, int max_blocks, int QB, int KB, int num_partial,
+                         int seqlen_orig, int dtype, void* stream);
 
 /*
  * Measurement aid (no counterpart in the reference): enqueue a kernel that issues nothing but

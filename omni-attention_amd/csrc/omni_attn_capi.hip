@@ -4,7 +4,7 @@
 // minus everything that is a property of torch tensors (dtype objects, contiguity),
 // which the binding layer above this file checks.
 #include "../../include/omni_attn_gfx950.h"
-#include "omni_attn_fwd_kernel.hpp"
+#include "omni_attn_bwd_kernel.hpp"
 
 #include <atomic>
 #include <cmath>
@@ -19,6 +19,14 @@ template <> int launch_fwd_blocks<false, 128>(const FwdParams&, int, int, hipStr
 template <> int launch_fwd_blocks<true, 32>(const FwdParams&, int, int, hipStream_t);
 template <> int launch_fwd_blocks<true, 64>(const FwdParams&, int, int, hipStream_t);
 template <> int launch_fwd_blocks<true, 128>(const FwdParams&, int, int, hipStream_t);
+template <bool BF16, int D>
+int launch_bwd_blocks(const BwdParams& p, int QB, int KB, hipStream_t stream);
+template <> int launch_bwd_blocks<false, 32>(const BwdParams&, int, int, hipStream_t);
+template <> int launch_bwd_blocks<false, 64>(const BwdParams&, int, int, hipStream_t);
+template <> int launch_bwd_blocks<false, 128>(const BwdParams&, int, int, hipStream_t);
+template <> int launch_bwd_blocks<true, 32>(const BwdParams&, int, int, hipStream_t);
+template <> int launch_bwd_blocks<true, 64>(const BwdParams&, int, int, hipStream_t);
+template <> int launch_bwd_blocks<true, 128>(const BwdParams&, int, int, hipStream_t);
 }  // namespace omni_attn
 
 namespace {
@@ -183,6 +191,108 @@ extern "C" int omni_attn_fwd_packed_gfx950(const void* q, const void* k, const v
                  seqlen_orig, dtype, stream);
 }
 
+extern "C" size_t omni_attn_bwd_workspace_bytes(int B, int H, int S_pad) {
+  if (B <= 0 || H <= 0 || S_pad <= 0) return 0;
+  return size_t(B) * size_t(H) * size_t(S_pad) * sizeof(float);  // delta = rowsum(dO . O)
+}
+
+namespace {
+// The backward with the workspace already chosen (caller's, or the library's static one).
+int backward(const void* q, const void* k, const void* v, const void* o, const void* dout,
+             const float* lse, void* dq, void* dk, void* dv, const int32_t* kv_num_blocks,
+             const int32_t* kv_indices, const int32_t* block_mask_types,
+             const int32_t* partial_idx_or_null, const uint8_t* partial_masks_or_null,
+             const uint32_t* partial_bits_or_null, float* delta_workspace, int B, int H, int S_pad,
+             int D, int Tq, int max_blocks, int QB, int KB, int num_partial, int seqlen_orig, int dtype,
+             void* stream) {
+  using namespace omni_attn;
+  if (!q || !k || !v || !o || !dout || !lse || !dq || !dk || !dv || !kv_num_blocks || !kv_indices ||
+      !block_mask_types || !delta_workspace)
+    return OMNI_ATTN_ERR_NULL_POINTER;
+  const auto misaligned = [](const void* ptr, uintptr_t a) { return (reinterpret_cast<uintptr_t>(ptr) & (a - 1)) != 0; };
+  if (misaligned(q, 16) || misaligned(k, 16) || misaligned(v, 16) || misaligned(o, 16) || misaligned(dout, 16) ||
+      misaligned(dq, 16) || misaligned(dk, 16) || misaligned(dv, 16) || misaligned(partial_masks_or_null, 16) ||
+      misaligned(partial_bits_or_null, 4) || misaligned(lse, 4) || misaligned(delta_workspace, 4) ||
+      misaligned(kv_num_blocks, 4) || misaligned(kv_indices, 4) || misaligned(block_mask_types, 4) ||
+      misaligned(partial_idx_or_null, 4))
+    return OMNI_ATTN_ERR_MISALIGNED;
+  if (dtype != OMNI_ATTN_DTYPE_F16 && dtype != OMNI_ATTN_DTYPE_BF16) return OMNI_ATTN_ERR_UNSUPPORTED_DTYPE;
+  if (D != 32 && D != 64 && D != 128) return OMNI_ATTN_ERR_UNSUPPORTED_HEAD_DIM;
+  if ((QB != 64 && QB != 128) || (KB != 64 && KB != 128)) return OMNI_ATTN_ERR_UNSUPPORTED_BLOCK;
+  if (B <= 0 || H <= 0 || S_pad <= 0 || Tq <= 0 || max_blocks <= 0 || seqlen_orig < 0 || num_partial < 0)
+    return OMNI_ATTN_ERR_BAD_SHAPE;
+  if (Tq != (S_pad + QB - 1) / QB) return OMNI_ATTN_ERR_BAD_SHAPE;
+  const long long total = (long long)B * H * Tq;
+  const int Tk = (S_pad + KB - 1) / KB;
+  if ((long long)S_pad * D > 0x7fffffffLL || total > 0x7fffffffLL / 2 || (long long)B * H * Tk > 0x7fffffffLL / 2 ||
+      total * max_blocks > (1LL << 40) || (long long)num_partial * QB * KB > 0x7fffffffLL * 64)
+    return OMNI_ATTN_ERR_TOO_LARGE;
+  // the dK/dV kernel keeps one bit per (query block, slot) of a slab in LDS
+  if ((long long)Tq * ((max_blocks + 63) / 64) > BwdDkdvTraits<128, 128>::kMaxBitmapWords)
+    return OMNI_ATTN_ERR_TOO_LARGE;
+
+  BwdParams p;
+  p.q = static_cast<const uint16_t*>(q);
+  p.k = static_cast<const uint16_t*>(k);
+  p.v = static_cast<const uint16_t*>(v);
+  p.o = static_cast<const uint16_t*>(o);
+  p.dout = static_cast<const uint16_t*>(dout);
+  p.lse = lse;
+  p.dq = static_cast<uint16_t*>(dq);
+  p.dk = static_cast<uint16_t*>(dk);
+  p.dv = static_cast<uint16_t*>(dv);
+  p.delta = delta_workspace;
+  p.kv_num_blocks = kv_num_blocks;
+  p.kv_indices = kv_indices;
+  p.types = block_mask_types;
+  const bool has_partial = partial_idx_or_null != nullptr && num_partial > 0 &&
+                           (partial_masks_or_null != nullptr || partial_bits_or_null != nullptr);
+  p.partial_idx = has_partial ? partial_idx_or_null : nullptr;
+  p.partial_masks = has_partial && partial_bits_or_null == nullptr ? partial_masks_or_null : nullptr;
+  p.partial_bits = has_partial ? partial_bits_or_null : nullptr;
+  p.num_partial = has_partial ? num_partial : 0;
+  p.S = S_pad;
+  p.Tq = Tq;
+  p.Tk = Tk;
+  p.max_blocks = max_blocks;
+  p.seqlen = seqlen_orig < S_pad ? seqlen_orig : S_pad;
+  p.n_slabs = B * H;
+  p.scale = float(1.0 / std::sqrt(double(D)));
+  p.sl2 = float(1.4426950408889634 / std::sqrt(double(D)));
+
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool bf = dtype == OMNI_ATTN_DTYPE_BF16;
+  int err;
+  switch (D) {
+    case 32: err = bf ? launch_bwd_blocks<true, 32>(p, QB, KB, s) : launch_bwd_blocks<false, 32>(p, QB, KB, s); break;
+    case 64: err = bf ? launch_bwd_blocks<true, 64>(p, QB, KB, s) : launch_bwd_blocks<false, 64>(p, QB, KB, s); break;
+    default: err = bf ? launch_bwd_blocks<true, 128>(p, QB, KB, s) : launch_bwd_blocks<false, 128>(p, QB, KB, s); break;
+  }
+  if (err != 0) {
+    g_last_hip_error = err;
+    return OMNI_ATTN_ERR_LAUNCH;
+  }
+  return OMNI_ATTN_OK;
+}
+}  // namespace
+
+extern "C" int omni_attn_bwd_gfx950(const void* q, const void* k, const void* v, const void* o,
+                                    const void* dout, const float* lse, void* dq, void* dk, void* dv,
+                                    const int32_t* kv_num_blocks, const int32_t* kv_indices,
+                                    const int32_t* block_mask_types, const int32_t* partial_idx_or_null,
+                                    const uint8_t* partial_masks_or_null,
+                                    const uint32_t* partial_bits_or_null, void* workspace,
+                                    size_t workspace_bytes, int B, int H, int S_pad, int D, int Tq,
+                                    int max_blocks, int QB, int KB, int num_partial, int seqlen_orig,
+                                    int dtype, void* stream) {
+  if (B > 0 && H > 0 && S_pad > 0 && workspace_bytes < omni_attn_bwd_workspace_bytes(B, H, S_pad))
+    return OMNI_ATTN_ERR_WORKSPACE;
+  return backward(q, k, v, o, dout, lse, dq, dk, dv, kv_num_blocks, kv_indices, block_mask_types,
+                  partial_idx_or_null, partial_masks_or_null, partial_bits_or_null,
+                  static_cast<float*>(workspace), B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial,
+                  seqlen_orig, dtype, stream);
+}
+
 extern "C" const char* omni_attn_status_string(int status) {
   switch (status) {
     case OMNI_ATTN_OK: return "ok";
@@ -194,6 +304,7 @@ extern "C" const char* omni_attn_status_string(int status) {
     case OMNI_ATTN_ERR_LAUNCH: return "HIP kernel launch failed";
     case OMNI_ATTN_ERR_TOO_LARGE: return "tensor too large for 32-bit slab indexing";
     case OMNI_ATTN_ERR_MISALIGNED: return "misaligned pointer: q, k, v, o and partial masks need 16 bytes, 32-bit arrays 4";
+    case OMNI_ATTN_ERR_WORKSPACE: return "workspace too small (see omni_attn_bwd_workspace_bytes)";
     default: return "unknown status";
   }
 }

@@ -200,6 +200,76 @@ void omni_attn_forward_packed(torch::Tensor Q, torch::Tensor K, torch::Tensor V,
                seqlen_orig, partial_block_mask_indices, partial_block_bits, true, true);
 }
 
+// Backward of omni_attn_forward: dQ, dK, dV written in place (the reference exports no backward).
+// PARTIAL tiles as bool bytes or, when `packed`, as the int32 words of omni_attn_pack_partial_masks.
+void omni_attn_backward(torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch::Tensor O,
+                        torch::Tensor dO, torch::Tensor LSE, torch::Tensor dQ, torch::Tensor dK,
+                        torch::Tensor dV, torch::Tensor kv_num_blocks, torch::Tensor kv_indices,
+                        torch::Tensor block_mask_types, int Q_BLOCK_SIZE, int KV_BLOCK_SIZE,
+                        int seqlen_orig, torch::Tensor partial_block_mask_indices,
+                        torch::Tensor partial_tiles, bool has_partial, bool packed) {
+  if (Q.scalar_type() != torch::kHalf && Q.scalar_type() != torch::kBFloat16)
+    throw std::runtime_error("Tensor dtype mismatch: Q must be torch.float16 or torch.bfloat16");
+  check_qkvo(Q, "Q", Q);
+  check_qkvo(K, "K", Q);
+  check_qkvo(V, "V", Q);
+  check_qkvo(O, "O", Q);
+  check_qkvo(dO, "dO", Q);
+  check_qkvo(dQ, "dQ", Q);
+  check_qkvo(dK, "dK", Q);
+  check_qkvo(dV, "dV", Q);
+  for (const torch::Tensor* t : {&Q, &K, &V, &O, &dO, &dQ, &dK, &dV})
+    if (!t->is_contiguous())
+      throw std::runtime_error("Q, K, V, O, dO, dQ, dK, dV tensors must be contiguous.");
+  check_meta(kv_num_blocks, "kv_num_blocks", Q);
+  check_meta(kv_indices, "kv_indices", Q);
+  check_meta(block_mask_types, "block_mask_types", Q);
+  if (!kv_num_blocks.is_contiguous() || !kv_indices.is_contiguous() || !block_mask_types.is_contiguous())
+    throw std::runtime_error("Block mask tensors must be contiguous.");
+  const int64_t B = Q.size(0), H = Q.size(1), S = Q.size(2), D = Q.size(3);
+  if (kv_num_blocks.dim() != 3 || kv_indices.dim() != 4 || block_mask_types.sizes() != kv_indices.sizes() ||
+      kv_num_blocks.size(0) != B || kv_num_blocks.size(1) != H || kv_indices.size(0) != B ||
+      kv_indices.size(1) != H || kv_indices.size(2) != kv_num_blocks.size(2))
+    throw std::runtime_error("Block mask tensor shapes do not match Q's batch / heads / blocks");
+  if (LSE.scalar_type() != torch::kFloat32 || !LSE.is_contiguous() || LSE.dim() != 3 || LSE.size(0) != B ||
+      LSE.size(1) != H || LSE.size(2) != S || LSE.device() != Q.device())
+    throw std::runtime_error("LSE must be the forward's contiguous fp32 [B, H, S] tensor on the device of Q");
+  const int32_t* pidx = nullptr;
+  const void* tiles = nullptr;
+  int num_partial = 0;
+  if (has_partial && partial_tiles.numel() > 0) {
+    if (partial_block_mask_indices.scalar_type() != torch::kInt32 ||
+        partial_block_mask_indices.sizes() != kv_indices.sizes() || !partial_block_mask_indices.is_contiguous() ||
+        partial_block_mask_indices.device() != Q.device())
+      throw std::runtime_error("partial_block_mask_indices must be a contiguous int32 tensor of the shape of kv_indices");
+    if (partial_tiles.scalar_type() != (packed ? torch::kInt32 : torch::kBool) || partial_tiles.dim() != 3 ||
+        partial_tiles.size(1) != Q_BLOCK_SIZE || partial_tiles.size(2) != (packed ? KV_BLOCK_SIZE / 32 : KV_BLOCK_SIZE) ||
+        !partial_tiles.is_contiguous() || partial_tiles.device() != Q.device())
+      throw std::runtime_error("partial tiles must be [num_partial, Q_BLOCK_SIZE, KV_BLOCK_SIZE] bool or packed int32 words");
+    pidx = partial_block_mask_indices.data_ptr<int32_t>();
+    tiles = partial_tiles.data_ptr();
+    num_partial = int(partial_tiles.size(0));
+  }
+  c10::DeviceGuard guard(Q.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStream(Q.device().index()).stream();
+  const size_t ws_bytes = omni_attn_bwd_workspace_bytes(int(B), int(H), int(S));
+  torch::Tensor workspace = torch::empty({int64_t(ws_bytes)}, Q.options().dtype(torch::kUInt8));
+  const int dtype = Q.scalar_type() == torch::kBFloat16 ? OMNI_ATTN_DTYPE_BF16 : OMNI_ATTN_DTYPE_F16;
+  const int rc = omni_attn_bwd_gfx950(
+      Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), dO.data_ptr(), LSE.data_ptr<float>(),
+      dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(), kv_num_blocks.data_ptr<int32_t>(),
+      kv_indices.data_ptr<int32_t>(), block_mask_types.data_ptr<int32_t>(), pidx,
+      packed ? nullptr : static_cast<const uint8_t*>(tiles), packed ? static_cast<const uint32_t*>(tiles) : nullptr,
+      workspace.data_ptr(), ws_bytes, int(B), int(H), int(S), int(D), int(kv_num_blocks.size(2)),
+      int(kv_indices.size(3)), Q_BLOCK_SIZE, KV_BLOCK_SIZE, num_partial, seqlen_orig, dtype,
+      static_cast<void*>(stream));
+  if (rc != OMNI_ATTN_OK) {
+    std::string msg = std::string("omni_attn: ") + omni_attn_status_string(rc);
+    if (rc == OMNI_ATTN_ERR_LAUNCH) msg += " (hipError " + std::to_string(omni_attn_last_hip_error()) + ")";
+    throw std::runtime_error(msg);
+  }
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -217,5 +287,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "omni_attn_pack_partial_masks (bool tiles -> 32-bit words)");
   m.def("omni_attn_forward_packed", &omni_attn_forward_packed,
         "omni_attn_forward_packed (PARTIAL tiles as packed words)");
+  m.def("omni_attn_backward", &omni_attn_backward, "omni_attn_backward (dQ, dK, dV of omni_attn_forward)");
   m.def("abi_version", []() { return omni_attn_abi_version(); });
 }

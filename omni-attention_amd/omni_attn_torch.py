@@ -482,7 +482,7 @@ _SUPPORTED_BLOCKS = (64, 128)
 
 def _omni_attention(op_name: str, query: Tensor, key: Tensor, value: Tensor,
                     block_mask: OmniBlockMask, partial_needs_partial_types: bool,
-                    return_lse: bool = False):
+                    return_lse: bool = False, keep_padded: bool = False):
     ext = _load_extension()
     B, H, Q, D = query.shape
     KV = key.shape[2]
@@ -556,6 +556,8 @@ def _omni_attention(op_name: str, query: Tensor, key: Tensor, value: Tensor,
         ext.omni_attn_forward_packed(query_padded, key_padded, value_padded, output_padded, lse_padded,
                                      kv_num_blocks, kv_indices, block_mask_types, QB, KB, q_orig_len,
                                      partial_idx, block_mask.partial_block_bits.contiguous())
+        if keep_padded:
+            return output_padded, lse_padded, query_padded, key_padded, value_padded, q_orig_len
         if return_lse:
             return output_padded[:, :, :q_orig_len, :], lse_padded[:, :, :q_orig_len]
         return output_padded[:, :, :q_orig_len, :]
@@ -564,6 +566,8 @@ def _omni_attention(op_name: str, query: Tensor, key: Tensor, value: Tensor,
         ext.omni_attn_forward(query_padded, key_padded, value_padded, output_padded, lse_padded,
                               kv_num_blocks, kv_indices, block_mask_types, QB, KB, q_orig_len,
                               partial_idx, partial_masks, has_partial)
+        if keep_padded:
+            return output_padded, lse_padded, query_padded, key_padded, value_padded, q_orig_len
         return output_padded[:, :, :q_orig_len, :], lse_padded[:, :, :q_orig_len]
     getattr(ext, op_name)(query_padded, key_padded, value_padded, output_padded,
                           kv_num_blocks, kv_indices, block_mask_types, QB, KB, q_orig_len,
@@ -607,6 +611,55 @@ def omni_attention_forward(query: Tensor, key: Tensor, value: Tensor,
     """Output and fp32 row logsumexp [B, H, S] (-inf for rows with no allowed key).
     Not in the reference, which has no logsumexp output."""
     return _omni_attention("omni_attn_forward", query, key, value, block_mask, False, return_lse=True)
+
+
+class _OmniAttentionFunction(torch.autograd.Function):
+    """Forward and backward kernels as one differentiable operator.  The reference's operator
+    cannot be differentiated (it has no backward and no logsumexp output); this is the form a
+    training loop needs, e.g. in place of the flex_attention call of
+    transfusion_pytorch/transfusion.py:953-983."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, block_mask):
+        out_padded, lse_padded, q_pad, k_pad, v_pad, seq_len = _omni_attention(
+            "omni_attn_forward", query, key, value, block_mask, False, return_lse=True, keep_padded=True)
+        ctx.save_for_backward(q_pad, k_pad, v_pad, out_padded, lse_padded)
+        ctx.block_mask = block_mask
+        ctx.seq_len = seq_len
+        return out_padded[:, :, :seq_len, :]
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        ext = _load_extension()
+        q_pad, k_pad, v_pad, out_padded, lse_padded = ctx.saved_tensors
+        m, seq_len = ctx.block_mask, ctx.seq_len
+        dev = q_pad.device
+        S_pad = q_pad.shape[2]
+        d_out = grad_out.to(q_pad.dtype)
+        if S_pad != seq_len:
+            d_out = F.pad(d_out, (0, 0, 0, S_pad - seq_len))
+        d_out = d_out.contiguous()
+        dq, dk, dv = torch.empty_like(q_pad), torch.empty_like(q_pad), torch.empty_like(q_pad)
+        to_i32 = lambda t: t.to(device=dev, dtype=torch.int32).contiguous()
+        has_partial = m.partial_block_mask_indices is not None and m.partial_block_masks is not None
+        packed = has_partial and m.partial_block_bits is not None and m.partial_block_bits.device == dev
+        if has_partial:
+            pidx = to_i32(m.partial_block_mask_indices)
+            tiles = (m.partial_block_bits.contiguous() if packed
+                     else m.partial_block_masks.to(device=dev, dtype=torch.bool).contiguous())
+        else:
+            pidx = torch.empty(0, dtype=torch.int32, device=dev)
+            tiles = torch.empty(0, dtype=torch.bool, device=dev)
+        ext.omni_attn_backward(q_pad, k_pad, v_pad, out_padded, d_out, lse_padded, dq, dk, dv,
+                               to_i32(m.kv_num_blocks), to_i32(m.kv_indices), to_i32(m.block_mask_types),
+                               m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, seq_len, pidx, tiles, has_partial, packed)
+        return dq[:, :, :seq_len, :], dk[:, :, :seq_len, :], dv[:, :, :seq_len, :], None
+
+
+def omni_attention(query: Tensor, key: Tensor, value: Tensor, block_mask: OmniBlockMask) -> Tensor:
+    """Differentiable block-sparse attention: the forward kernel, with the backward kernels
+    behind ``.backward()`` (gradients with respect to query, key and value)."""
+    return _OmniAttentionFunction.apply(query, key, value, block_mask)
 
 
 # ----------------------------------------------------------------------------

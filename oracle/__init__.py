@@ -21,6 +21,10 @@ How each is pinned (tests/test_oracle_pinning.py):
     (omni-attn-mma/logs/printed_mask.md:3-57, :59-76, :123-139, :153-176), held as data in
     tests/golden/printed_masks.json.
   * the two restatements against each other on random metadata.
+  * gradients (dense_oracle.attention_dense_grads: autograd through the dense oracle, for the
+    backward kernels, which have no counterpart in the reference): torch.autograd.gradcheck in
+    fp64 on tiny inputs, the textbook closed form written without autograd, and the special
+    case of one allowed key per row (dV = scatter of dO, dQ = dK = 0).
 The reference's own golden tensors (*.pt) are absent from its tree, and its CUDA sources
 cannot be compiled here (mma.sync / cp.async PTX), so there is no oracle/_ref build.
 """

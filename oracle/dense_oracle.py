@@ -37,6 +37,48 @@ def attention_dense_fp32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     return out, lse
 
 
+def attention_dense_differentiable(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                                   mask: torch.Tensor) -> torch.Tensor:
+    """The same function as attention_dense_fp32 (output only) written so that autograd can
+    go through it, in the dtype of its inputs (fp32, or fp64 for gradcheck): rows with no
+    allowed key give 0 and pass no gradient."""
+    D = q.shape[-1]
+    s = torch.matmul(q, k.transpose(-1, -2)) / math.sqrt(D)
+    any_row = mask.any(-1, keepdim=True)
+    s = s.masked_fill(~mask, float("-inf"))
+    s = torch.where(any_row, s, torch.zeros_like(s))  # keeps softmax finite on empty rows
+    p = torch.softmax(s, dim=-1)
+    p = torch.where(any_row, p, torch.zeros_like(p))
+    return torch.matmul(p, v)
+
+
+def attention_dense_grads(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor,
+                          dout: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dQ, dK, dV) of sum(O * dout) by autograd through attention_dense_differentiable in fp32
+    (inputs of any float dtype are converted as they are)."""
+    qf, kf, vf = (t.detach().float().clone().requires_grad_(True) for t in (q, k, v))
+    out = attention_dense_differentiable(qf, kf, vf, mask)
+    out.backward(dout.float())
+    return qf.grad, kf.grad, vf.grad
+
+
+def attention_dense_grads_closed_form(q, k, v, mask, dout):
+    """The textbook closed form, written out with no autograd: P = softmax(mask(QK^T/sqrt(D))),
+    delta_i = sum_d dO_id O_id, dV = P^T dO, dS = P * (dO V^T - delta), dQ = dS K / sqrt(D),
+    dK = dS^T Q / sqrt(D).  Pins attention_dense_grads (and is pinned by gradcheck with it)."""
+    qf, kf, vf, do = q.float(), k.float(), v.float(), dout.float()
+    scale = 1.0 / math.sqrt(qf.shape[-1])
+    s = torch.matmul(qf, kf.transpose(-1, -2)) * scale
+    any_row = mask.any(-1, keepdim=True)
+    s = torch.where(any_row, s.masked_fill(~mask, float("-inf")), torch.zeros_like(s))
+    p = torch.where(any_row, torch.softmax(s, dim=-1), torch.zeros_like(s))
+    o = torch.matmul(p, vf)
+    delta = (do * o).sum(-1, keepdim=True)
+    dv = torch.matmul(p.transpose(-1, -2), do)
+    ds = p * (torch.matmul(do, vf.transpose(-1, -2)) - delta)
+    return torch.matmul(ds, kf) * scale, torch.matmul(ds.transpose(-1, -2), qf) * scale, dv
+
+
 def prefix_mask(prefix_len: torch.Tensor, kv_len: int) -> torch.Tensor:
     """allow[..., i, j] = j < prefix_len[..., i]."""
     j = torch.arange(kv_len, device=prefix_len.device)

@@ -1,0 +1,175 @@
+"""Parity of the backward kernels with autograd through the fp32 dense oracle, through the C ABI.
+
+The reference has no backward and north_star states no bar for gradients.  The bars used here:
+each gradient tensor is compared on the inputs the kernels saw (q, k, v, dO already rounded to
+the 16-bit type), normalised by the largest reference entry of that tensor:
+    max|d - d_ref| <= TOL * max(1, max|d_ref|),   TOL = 4e-3 (fp16), 3e-2 (bf16)
+(the kernels round P and dS to the 16-bit type before the second products of a step, as the
+forward rounds P: 2^-11 resp. 2^-8 relative per term).  Rows and keys beyond the sequence, and
+keys nobody attends, get exactly zero.
+"""
+import pytest
+import torch
+
+import omni_attn_capi
+from baseline_configs import make_workload
+from helpers import random_block_metadata
+from oracle.dense_oracle import attention_dense_grads, dense_mask_from_blocks, prefix_mask
+
+pytestmark = pytest.mark.gpu
+
+TOL_GRAD = {torch.float16: 4e-3, torch.bfloat16: 3e-2}
+
+
+def run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, seqlen, pidx=None, pm=None, device="cuda:0", packed=False):
+    dev = lambda t: None if t is None else t.to(device).contiguous()
+    qd, kd, vd, dod = dev(q), dev(k), dev(v), dev(dout)
+    nbd, idxd, tysd, pidxd, pmd = dev(nb), dev(idx), dev(tys), dev(pidx), dev(pm)
+    bits = omni_attn_capi.pack_partial_masks(pmd) if (packed and pmd is not None) else None
+    o = torch.full_like(qd, float("nan"))
+    lse = torch.full(qd.shape[:3], float("nan"), dtype=torch.float32, device=device)
+    if bits is not None:
+        omni_attn_capi.fwd(qd, kd, vd, o, lse, nbd, idxd, tysd, QB, KB, seqlen, pidxd, None, partial_bits=bits)
+    else:
+        omni_attn_capi.fwd(qd, kd, vd, o, lse, nbd, idxd, tysd, QB, KB, seqlen, pidxd, pmd)
+    dq, dk, dv = (torch.full_like(qd, float("nan")) for _ in range(3))
+    omni_attn_capi.bwd(qd, kd, vd, o, dod, lse, dq, dk, dv, nbd, idxd, tysd, QB, KB, seqlen, pidxd,
+                       None if bits is not None else pmd, bits)
+    torch.cuda.synchronize()
+    return dq, dk, dv, o, lse
+
+
+def check_grads(got, ref, dtype, what):
+    for name, a, b in zip(("dQ", "dK", "dV"), got, ref):
+        a = a.float().cpu()
+        assert torch.isfinite(a).all(), f"{what}: non-finite {name}"
+        err = (a - b).abs().max().item()
+        bar = TOL_GRAD[dtype] * max(1.0, b.abs().max().item())
+        assert err <= bar, f"{what}: max|d{name}| error {err:.3e} > {bar:.3e} (max|ref| {b.abs().max().item():.3f})"
+
+
+def test_c1_causal_backward(gpu_device):
+    w = make_workload("c1_causal", seed=0)
+    m = w.block_mask
+    gen = torch.Generator().manual_seed(100)
+    dout = torch.randn(w.q.shape, generator=gen).to(w.dtype)
+    S = w.q.shape[2]
+    got = run_fwd_bwd(w.q, w.k, w.v, dout, m.kv_num_blocks, m.kv_indices, m.block_mask_types, 128, 128, S,
+                      device=gpu_device)
+    ref = attention_dense_grads(w.q, w.k, w.v, prefix_mask(w.prefix_len, S).unsqueeze(1), dout)
+    check_grads(got[:3], ref, w.dtype, "c1")
+
+
+@pytest.mark.parametrize("packed", [False, True], ids=["bytes", "bits"])
+def test_c3_partial_shrunk_backward(packed, gpu_device):
+    w = make_workload("c3_partial", seed=2, H=2, S=2048)
+    m = w.block_mask
+    gen = torch.Generator().manual_seed(101)
+    dout = torch.randn(w.q.shape, generator=gen).to(w.dtype)
+    S = w.q.shape[2]
+    got = run_fwd_bwd(w.q, w.k, w.v, dout, m.kv_num_blocks, m.kv_indices, m.block_mask_types, m.Q_BLOCK_SIZE,
+                      m.KV_BLOCK_SIZE, S, m.partial_block_mask_indices, m.partial_block_masks,
+                      device=gpu_device, packed=packed)
+    ref = attention_dense_grads(w.q, w.k, w.v, prefix_mask(w.prefix_len, S).unsqueeze(1), dout)
+    check_grads(got[:3], ref, w.dtype, "c3 shrunk")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("QB,KB", [(128, 128), (128, 64), (64, 128), (64, 64)])
+def test_random_metadata_backward(dtype, D, QB, KB, gpu_device):
+    gen = torch.Generator().manual_seed(7000 + 10 * D + QB + KB // 64)
+    B, H, S = 2, 2, 512
+    q, k, v, dout = (torch.randn(B, H, S, D, generator=gen).to(dtype) for _ in range(4))
+    nb, idx, tys, pidx, pm = random_block_metadata(gen, B, H, S // QB, S // KB, QB, KB, shuffle=True)
+    for seqlen in (S, S - 45):
+        got = run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, seqlen, pidx, pm, device=gpu_device)
+        dense = dense_mask_from_blocks(nb, idx, tys, QB, KB, S, S, pidx, pm, seqlen_orig=seqlen)
+        ref = attention_dense_grads(q, k, v, dense, dout)
+        check_grads(got[:3], ref, dtype, f"random metadata seqlen={seqlen}")
+        for t in got[:3]:
+            assert (t[:, :, seqlen:] == 0).all(), "rows beyond the sequence must get zero gradients"
+
+
+def test_c2_full_size_backward_on_sampled_slabs(gpu_device):
+    w = make_workload("c2_interleaved", seed=0)
+    m = w.block_mask
+    B, H, S, D = w.q.shape
+    gen = torch.Generator().manual_seed(102)
+    dout = torch.randn(w.q.shape, generator=gen).to(w.dtype)
+    got = run_fwd_bwd(w.q, w.k, w.v, dout, m.kv_num_blocks, m.kv_indices, m.block_mask_types, 128, 128, S,
+                      device=gpu_device)
+    cpu = [t.float().cpu() for t in got[:3]]
+    for b, h in ((0, 0), (1, 17), (1, 31)):
+        mask = prefix_mask(w.prefix_len[b], S)
+        ref = attention_dense_grads(w.q[b, h], w.k[b, h], w.v[b, h], mask, dout[b, h])
+        check_grads([t[b, h] for t in cpu], ref, w.dtype, f"c2 slab ({b},{h})")
+
+
+def test_duplicate_and_clamped_block_indices_backward(gpu_device):
+    """The forward clamps block indices and visits a block as often as it is listed; the backward
+    differentiates exactly that (a block listed twice counts twice in the softmax)."""
+    gen = torch.Generator().manual_seed(103)
+    S, D = 256, 64
+    q, k, v, dout = (torch.randn(1, 1, S, D, generator=gen).to(torch.float16) for _ in range(4))
+    nb = torch.tensor([[[2, 3]]], dtype=torch.int32)
+    idx = torch.tensor([[[[0, 99, 0], [-5, 1, 1]]]], dtype=torch.int32)  # 99 -> 1, -5 -> 0; row 1 lists block 1 twice
+    tys = torch.full((1, 1, 2, 3), 2, dtype=torch.int32)
+    got = run_fwd_bwd(q, k, v, dout, nb, idx, tys, 128, 128, S, device=gpu_device)
+    # reference: keys of a twice-listed block appear twice
+    kk = torch.cat([k, k[:, :, 128:]], dim=2)
+    vv = torch.cat([v, v[:, :, 128:]], dim=2)
+    mask = torch.zeros(S, S + 128, dtype=torch.bool)
+    mask[:128, :256] = True
+    mask[128:, :] = True
+    dq, dkk, dvv = attention_dense_grads(q[0, 0], kk[0, 0], vv[0, 0], mask, dout[0, 0])
+    dk = dkk[:256].clone(); dk[128:] += dkk[256:]
+    dv = dvv[:256].clone(); dv[128:] += dvv[256:]
+    check_grads([t[0, 0] for t in got[:3]], (dq, dk, dv), torch.float16, "duplicates")
+
+
+def test_backward_is_bitwise_reproducible_and_checks_its_workspace(gpu_device):
+    w = make_workload("c3_partial", seed=5, H=2, S=1024)
+    m = w.block_mask
+    gen = torch.Generator().manual_seed(104)
+    dout = torch.randn(w.q.shape, generator=gen).to(w.dtype)
+    args = (w.q, w.k, w.v, dout, m.kv_num_blocks, m.kv_indices, m.block_mask_types, m.Q_BLOCK_SIZE,
+            m.KV_BLOCK_SIZE, 1024, m.partial_block_mask_indices, m.partial_block_masks)
+    a = run_fwd_bwd(*args, device=gpu_device)
+    b = run_fwd_bwd(*args, device=gpu_device)
+    for x, y in zip(a[:3], b[:3]):
+        assert torch.equal(x, y)
+    lib = omni_attn_capi.load_library()
+    assert lib.omni_attn_bwd_workspace_bytes(1, 2, 1024) == 1 * 2 * 1024 * 4
+    small = torch.empty(16, dtype=torch.uint8, device=gpu_device)
+    q = w.q.to(gpu_device)
+    with pytest.raises(RuntimeError, match="workspace"):
+        omni_attn_capi.bwd(q, q, q, q, q, torch.zeros(q.shape[:3], device=gpu_device), q.clone(), q.clone(), q.clone(),
+                           m.kv_num_blocks.to(gpu_device), m.kv_indices.to(gpu_device),
+                           m.block_mask_types.to(gpu_device), m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, 1024,
+                           workspace=small)
+
+
+def test_autograd_operator_matches_oracle_gradients(gpu_device):
+    """omni_attn_torch.omni_attention: forward + backward kernels behind torch.autograd, on a
+    sequence that is not a multiple of the block (the wrapper pads, gradients of padding are dropped)."""
+    import omni_attn_torch as oat
+    from omni_attn_torch import create_omni_block_mask_from_prefix_lengths, modality_prefix_lengths
+    gen = torch.Generator().manual_seed(105)
+    B, H, S, D = 1, 2, 500, 64
+    S_pad = 512
+    mp = torch.tensor([[[1, 100, 150], [1, 300, 90]]], dtype=torch.long)
+    prefix = modality_prefix_lengths(mp, S_pad)
+    mask = create_omni_block_mask_from_prefix_lengths(prefix, H, S_pad, S_pad, 128, 128)
+    q, k, v = (torch.randn(B, H, S, D, generator=gen).to(torch.bfloat16) for _ in range(3))
+    dout = torch.randn(B, H, S, D, generator=gen).to(torch.bfloat16)
+    qd, kd, vd = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v))
+    for m in (mask.to(gpu_device), mask.to(gpu_device).pack_partial_masks()):
+        for t in (qd, kd, vd):
+            t.grad = None
+        out = oat.omni_attention(qd, kd, vd, m)
+        assert out.shape == (B, H, S, D)
+        out.backward(dout.to(gpu_device))
+        dense = prefix_mask(prefix[:, :S], S_pad)[..., :S].unsqueeze(1)
+        ref = attention_dense_grads(q, k, v, dense, dout)
+        check_grads((qd.grad, kd.grad, vd.grad), ref, torch.bfloat16, "autograd operator")

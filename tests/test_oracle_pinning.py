@@ -221,3 +221,43 @@ def test_bitless_partial_slot_is_skipped_by_the_walk():
     tys_skip = torch.tensor([[[[1, 0], [0, 1]]]], dtype=torch.int32)
     o2, lse2 = attention_block_walk(q, k, v, nb, idx, tys_skip, 128, 128, 256)
     assert torch.equal(o, o2) and torch.equal(lse, lse2)
+
+
+# ---- gradients (oracle of the backward kernels) ------------------------------------------------
+
+def test_gradient_oracle_gradcheck_and_closed_form():
+    from oracle.dense_oracle import (attention_dense_differentiable, attention_dense_grads,
+                                     attention_dense_grads_closed_form)
+    gen = torch.Generator().manual_seed(31)
+    S, D = 7, 4
+    mask = torch.rand(2, S, S, generator=gen) < 0.6
+    mask[0, 3] = False  # a row with no allowed key: zero output, no gradient
+    q, k, v = (torch.randn(2, S, D, generator=gen, dtype=torch.float64, requires_grad=True) for _ in range(3))
+    assert torch.autograd.gradcheck(lambda a, b, c: attention_dense_differentiable(a, b, c, mask), (q, k, v),
+                                    eps=1e-6, atol=1e-6)
+    dout = torch.randn(2, S, D, generator=gen)
+    g_auto = attention_dense_grads(q, k, v, mask, dout)
+    g_form = attention_dense_grads_closed_form(q, k, v, mask, dout)
+    for a, b in zip(g_auto, g_form):
+        assert torch.allclose(a, b, atol=2e-6), (a - b).abs().max()
+    assert (g_auto[0][0, 3] == 0).all()  # the empty row passes nothing to its query
+    # the forward of the differentiable form is the oracle's forward
+    o_ref, _ = attention_dense_fp32(q.detach(), k.detach(), v.detach(), mask)
+    assert torch.allclose(attention_dense_differentiable(q.detach().float(), k.detach().float(),
+                                                         v.detach().float(), mask), o_ref, atol=1e-6)
+
+
+def test_gradient_oracle_one_allowed_key_per_row():
+    """With one allowed key per row the output is that V row whatever Q and K are:
+    dQ = dK = 0 and dV[j] = sum of dO over the rows that attend key j."""
+    from oracle.dense_oracle import attention_dense_grads
+    gen = torch.Generator().manual_seed(32)
+    S, D = 9, 8
+    target = torch.randint(0, S, (S,), generator=gen)
+    mask = torch.zeros(S, S, dtype=torch.bool)
+    mask[torch.arange(S), target] = True
+    q, k, v, dout = (torch.randn(S, D, generator=gen) for _ in range(4))
+    dq, dk, dv = attention_dense_grads(q, k, v, mask, dout)
+    assert dq.abs().max() < 1e-6 and dk.abs().max() < 1e-6
+    expect = torch.zeros(S, D).index_add_(0, target, dout)
+    assert torch.allclose(dv, expect, atol=1e-6)
