@@ -50,7 +50,9 @@ enum omni_attn_status {
   OMNI_ATTN_ERR_TOO_LARGE = 7,         /* a tensor exceeds 2^31-1 elements per (b,h) slab */
   OMNI_ATTN_ERR_MISALIGNED = 8,        /* q, k, v, o or partial masks not 16-byte aligned, or a
                                           32-bit array not 4-byte aligned */
-  OMNI_ATTN_ERR_WORKSPACE = 9          /* workspace smaller than omni_attn_bwd_workspace_bytes() */
+  OMNI_ATTN_ERR_WORKSPACE = 9,         /* workspace smaller than omni_attn_bwd_workspace_bytes() */
+  OMNI_ATTN_ERR_SCRATCH_LIMIT = 10     /* omni_attn_bwd_noalloc_gfx950: B * H * S_pad beyond its
+                                          built-in scratch (omni_attn_bwd_noalloc_max_rows()) */
 };
 
 /*
@@ -168,6 +170,30 @@ int omni_attn_bwd_gfx950(const void* q, const void* k, const void* v, const void
                          int B, int H, int S_pad, int D,
                          int Tq, int max_blocks, int QB, int KB, int num_partial,
                          int seqlen_orig, int dtype, void* stream);
+
+/*
+ * omni_attn_bwd_gfx950 for callers that cannot allocate device memory for the workspace: code
+ * under HIP graph capture, tight serving or training loops, harnesses that forbid allocation.
+ * No counterpart in the reference.  Same kernels and bit-identical results; the workspace is a
+ * 16 MiB device array built into the library (each GPU the library runs on holds its copy until
+ * the process ends), so B * H * S_pad must not exceed omni_attn_bwd_noalloc_max_rows()
+ * (4 194 304), else OMNI_ATTN_ERR_SCRATCH_LIMIT.  Calls no hipMalloc / hipFree or any other
+ * allocating routine.  All calls on one GPU share that GPU's array: calls that overlap in time
+ * on one GPU (different streams, different threads) race and must be serialised by the caller.
+ */
+size_t omni_attn_bwd_noalloc_max_rows(void);
+int omni_attn_bwd_noalloc_gfx950(const void* q, const void* k, const void* v, const void* o,
+                                 const void* dout, const float* lse,
+                                 void* dq, void* dk, void* dv,
+                                 const int32_t* kv_num_blocks,
+                                 const int32_t* kv_indices,
+                                 const int32_t* block_mask_types,
+                                 const int32_t* partial_idx_or_null,
+                                 const uint8_t* partial_masks_or_null,
+                                 const uint32_t* partial_bits_or_null,
+                                 int B, int H, int S_pad, int D,
+                                 int Tq, int max_blocks, int QB, int KB, int num_partial,
+                                 int seqlen_orig, int dtype, void* stream);
 
 /*
  * Measurement aid (no counterpart in the reference): enqueue a kernel that issues nothing but

@@ -293,6 +293,62 @@ extern "C" int omni_attn_bwd_gfx950(const void* q, const void* k, const void* v,
                   seqlen_orig, dtype, stream);
 }
 
+// ---- the backward for callers that cannot allocate -------------------------------------------
+// Same kernels; the delta workspace is this file-scope device array instead of caller memory.
+// Every GPU the library runs on holds its own copy at its own address until the process ends.
+constexpr size_t kScratchFloats = size_t(4) << 20;  // 16 MiB: B * H * S_pad up to 4 194 304 rows
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+namespace {
+float* g_scratch_ptr[kMaxDevices];
+std::atomic<bool> g_scratch_known[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up once per device: in host code the
+// array's name is only a handle for this lookup, never an address a kernel can use).
+int scratch_address(float** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return int(e);
+  if (dev < 0 || dev >= kMaxDevices) return int(hipErrorInvalidDevice);
+  if (!g_scratch_known[dev].load(std::memory_order_acquire)) {
+    float* ptr = nullptr;
+    e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return int(e);
+    if (ptr == nullptr) return int(hipErrorInvalidSymbol);
+    g_scratch_ptr[dev] = ptr;
+    g_scratch_known[dev].store(true, std::memory_order_release);
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+}  // namespace
+
+extern "C" size_t omni_attn_bwd_noalloc_max_rows(void) { return kScratchFloats; }
+
+extern "C" int omni_attn_bwd_noalloc_gfx950(const void* q, const void* k, const void* v, const void* o,
+                                            const void* dout, const float* lse, void* dq, void* dk,
+                                            void* dv, const int32_t* kv_num_blocks,
+                                            const int32_t* kv_indices, const int32_t* block_mask_types,
+                                            const int32_t* partial_idx_or_null,
+                                            const uint8_t* partial_masks_or_null,
+                                            const uint32_t* partial_bits_or_null, int B, int H, int S_pad,
+                                            int D, int Tq, int max_blocks, int QB, int KB, int num_partial,
+                                            int seqlen_orig, int dtype, void* stream) {
+  if (B <= 0 || H <= 0 || S_pad <= 0) return OMNI_ATTN_ERR_BAD_SHAPE;
+  if ((unsigned long long)B * (unsigned long long)H * (unsigned long long)S_pad > kScratchFloats)
+    return OMNI_ATTN_ERR_SCRATCH_LIMIT;
+  float* delta = nullptr;
+  if (const int e = scratch_address(&delta)) {
+    g_last_hip_error = e;
+    return OMNI_ATTN_ERR_LAUNCH;
+  }
+  // Nothing in the array has to start at zero: the dQ kernel writes delta for every row of every
+  // slab before the dK/dV kernel, which runs after it on the same stream, reads any of them.
+  return backward(q, k, v, o, dout, lse, dq, dk, dv, kv_num_blocks, kv_indices, block_mask_types,
+                  partial_idx_or_null, partial_masks_or_null, partial_bits_or_null, delta, B, H, S_pad, D,
+                  Tq, max_blocks, QB, KB, num_partial, seqlen_orig, dtype, stream);
+}
+
 extern "C" const char* omni_attn_status_string(int status) {
   switch (status) {
     case OMNI_ATTN_OK: return "ok";
@@ -305,6 +361,9 @@ extern "C" const char* omni_attn_status_string(int status) {
     case OMNI_ATTN_ERR_TOO_LARGE: return "tensor too large for 32-bit slab indexing";
     case OMNI_ATTN_ERR_MISALIGNED: return "misaligned pointer: q, k, v, o and partial masks need 16 bytes, 32-bit arrays 4";
     case OMNI_ATTN_ERR_WORKSPACE: return "workspace too small (see omni_attn_bwd_workspace_bytes)";
+    case OMNI_ATTN_ERR_SCRATCH_LIMIT:
+      return "B * H * S_pad exceeds the built-in scratch of omni_attn_bwd_noalloc_gfx950 (4 194 304 rows); "
+             "use omni_attn_bwd_gfx950 with a workspace";
     default: return "unknown status";
   }
 }

@@ -23,6 +23,8 @@ EXPORTED_SYMBOLS = (
     "omni_attn_pack_partial_masks_gfx950",
     "omni_attn_bwd_gfx950",
     "omni_attn_bwd_workspace_bytes",
+    "omni_attn_bwd_noalloc_gfx950",
+    "omni_attn_bwd_noalloc_max_rows",
     "omni_attn_mfma_peak_probe_gfx950",
     "omni_attn_status_string",
     "omni_attn_last_hip_error",
@@ -47,6 +49,9 @@ def load_library() -> ctypes.CDLL:
         lib.omni_attn_bwd_workspace_bytes.argtypes = [i32, i32, i32]
         lib.omni_attn_bwd_gfx950.restype = i32
         lib.omni_attn_bwd_gfx950.argtypes = [vp] * 16 + [ctypes.c_size_t] + [i32] * 11 + [vp]
+        lib.omni_attn_bwd_noalloc_max_rows.restype = ctypes.c_size_t
+        lib.omni_attn_bwd_noalloc_gfx950.restype = i32
+        lib.omni_attn_bwd_noalloc_gfx950.argtypes = [vp] * 15 + [i32] * 11 + [vp]
         lib.omni_attn_mfma_peak_probe_gfx950.restype = i32
         lib.omni_attn_mfma_peak_probe_gfx950.argtypes = [i32, i32, vp, ctypes.POINTER(ctypes.c_double), vp]
         lib.omni_attn_status_string.restype = ctypes.c_char_p
@@ -157,11 +162,12 @@ def fwd(q, k, v, o, lse, kv_num_blocks, kv_indices, block_mask_types, QB, KB, se
 
 def bwd(q, k, v, o, dout, lse, dq, dk, dv, kv_num_blocks, kv_indices, block_mask_types, QB, KB, seqlen_orig,
         partial_idx=None, partial_masks=None, partial_bits=None, workspace: Optional[torch.Tensor] = None,
-        stream: Optional[int] = None) -> None:
+        stream: Optional[int] = None, no_alloc: bool = False) -> None:
     """Enqueue the backward (two kernels) on ``stream``.  All of q, k, v, o, dout, dq, dk, dv are
     contiguous [B, H, S_pad, D] GPU tensors of one 16-bit dtype, lse is the forward's fp32
     [B, H, S_pad].  ``workspace``: a GPU tensor of at least omni_attn_bwd_workspace_bytes bytes
-    (allocated here, by torch, when not given)."""
+    (allocated here, by torch, when not given).  ``no_alloc=True`` calls omni_attn_bwd_noalloc_gfx950
+    instead: no workspace, the library's built-in scratch."""
     B, H, S, D = q.shape
     for t in (q, k, v, o, dout, dq, dk, dv):
         if not (t.is_cuda and t.is_contiguous() and t.dtype == q.dtype and t.shape == q.shape):
@@ -175,10 +181,12 @@ def bwd(q, k, v, o, dout, lse, dq, dk, dv, kv_num_blocks, kv_indices, block_mask
     if not (lse.is_cuda and lse.is_contiguous() and lse.dtype == torch.float32 and lse.shape == q.shape[:3]):
         raise RuntimeError("lse must be the forward's contiguous fp32 [B, H, S_pad] tensor")
     lib = load_library()
-    need = lib.omni_attn_bwd_workspace_bytes(B, H, S)
-    if workspace is None:
-        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
-    ws_bytes = workspace.numel() * workspace.element_size()
+    ws_bytes = 0
+    if not no_alloc:
+        need = lib.omni_attn_bwd_workspace_bytes(B, H, S)
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        ws_bytes = workspace.numel() * workspace.element_size()
     num_partial = 0
     if partial_bits is not None:
         num_partial = int(partial_bits.shape[0])
@@ -188,6 +196,17 @@ def bwd(q, k, v, o, dout, lse, dq, dk, dv, kv_num_blocks, kv_indices, block_mask
         partial_idx = partial_masks = partial_bits = None
     if stream is None:
         stream = torch.cuda.current_stream(q.device).cuda_stream
+    if no_alloc:
+        with torch.cuda.device(q.device):
+            rc = lib.omni_attn_bwd_noalloc_gfx950(
+                _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(dout), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv),
+                _ptr(kv_num_blocks), _ptr(kv_indices), _ptr(block_mask_types), _ptr(partial_idx),
+                _ptr(partial_masks if partial_bits is None else None), _ptr(partial_bits),
+                B, H, S, D, kv_num_blocks.shape[2], kv_indices.shape[3], QB, KB, num_partial, int(seqlen_orig),
+                dtype, stream)
+        if rc != 0:
+            raise RuntimeError("omni_attn_bwd_noalloc_gfx950: %s (status %d)" % (status_string(rc), rc))
+        return
     with torch.cuda.device(q.device):
         rc = lib.omni_attn_bwd_gfx950(
             _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(dout), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv),
