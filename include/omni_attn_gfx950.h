@@ -86,6 +86,11 @@ enum omni_attn_status {
  *   Tq               number of query blocks, must equal ceil(S_pad / QB).
  *   seqlen_orig      rows >= seqlen_orig are written as zeros (lse -inf); keys
  *                    >= seqlen_orig are never attended (attn_naive.cu:64-72, :113).
+ *   softcap          0 = off (the reference's operator).  > 0: the scaled score x = q.k / sqrt(D)
+ *                    is replaced by softcap * tanh(x / softcap) before the mask and the softmax,
+ *                    the score_mod Transfusion's attention layer passes to flex_attention
+ *                    (transfusion_pytorch/transfusion.py:358-364, :958-959).  Negative, NaN or
+ *                    infinite values are refused (OMNI_ATTN_ERR_BAD_SHAPE).
  *
  * Semantics per slot: MASKED is skipped; FULL keeps everything; CAUSAL keeps
  * k_global <= q_global; PARTIAL keeps the stored bytes; a PARTIAL slot whose
@@ -107,7 +112,7 @@ int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v, void* o,
                          const uint8_t* partial_masks_or_null,
                          int B, int H, int S_pad, int D,
                          int Tq, int max_blocks, int QB, int KB, int num_partial,
-                         int seqlen_orig, int dtype, void* stream);
+                         int seqlen_orig, int dtype, float softcap, void* stream);
 
 /*
  * Pre-pass for masks that are reused over many launches: packs the bool tiles that the
@@ -134,7 +139,7 @@ int omni_attn_fwd_packed_gfx950(const void* q, const void* k, const void* v, voi
                                 const uint32_t* partial_bits_or_null,
                                 int B, int H, int S_pad, int D,
                                 int Tq, int max_blocks, int QB, int KB, int num_partial,
-                                int seqlen_orig, int dtype, void* stream);
+                                int seqlen_orig, int dtype, float softcap, void* stream);
 
 /*
  * Backward of omni_attn_fwd_gfx950: gradients of a scalar loss with respect to q, k and v,
@@ -169,7 +174,7 @@ int omni_attn_bwd_gfx950(const void* q, const void* k, const void* v, const void
                          void* workspace, size_t workspace_bytes,
                          int B, int H, int S_pad, int D,
                          int Tq, int max_blocks, int QB, int KB, int num_partial,
-                         int seqlen_orig, int dtype, void* stream);
+                         int seqlen_orig, int dtype, float softcap, void* stream);
 
 /*
  * omni_attn_bwd_gfx950 for callers that cannot allocate device memory for the workspace: code
@@ -193,7 +198,7 @@ int omni_attn_bwd_noalloc_gfx950(const void* q, const void* k, const void* v, co
                                  const uint32_t* partial_bits_or_null,
                                  int B, int H, int S_pad, int D,
                                  int Tq, int max_blocks, int QB, int KB, int num_partial,
-                                 int seqlen_orig, int dtype, void* stream);
+                                 int seqlen_orig, int dtype, float softcap, void* stream);
 
 /*
  * Measurement aid (no counterpart in the reference): enqueue a kernel that issues nothing but
@@ -212,7 +217,7 @@ const char* omni_attn_status_string(int status);
 /* hipError_t of the most recent failed launch on the calling thread (0 if none). */
 int omni_attn_last_hip_error(void);
 
-/* Version of this ABI; bumped when a signature changes (2: num_partial added). */
+/* Version of this ABI; bumped when a signature changes (2: num_partial added; 3: softcap added). */
 int omni_attn_abi_version(void);
 
 #ifdef __cplusplus

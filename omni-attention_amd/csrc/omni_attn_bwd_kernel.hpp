@@ -49,9 +49,26 @@ struct BwdParams {
   const uint32_t* partial_bits;
   int num_partial;
   int S, Tq, Tk, max_blocks, seqlen, n_slabs;
-  float sl2;    // log2(e) / sqrt(D)
-  float scale;  // 1 / sqrt(D)
+  float sl2;      // log2(e) / sqrt(D)
+  float scale;    // 1 / sqrt(D)
+  float softcap;  // > 0: the forward replaced x = s / sqrt(D) by softcap * tanh(x / softcap)
+  float cap_c2;   // 2 * log2(e) / (sqrt(D) * softcap)
 };
+
+// Weight and score-gradient factor of one score.  Plain: p = exp2(s * sl2 - lse2), factor 1.
+// Soft-capped: t = tanh(s / sqrt(D) / cap), p = exp2(cap * t * log2 e - lse2), factor 1 - t^2
+// (the derivative of cap * tanh(x / cap) with respect to x).
+__device__ __forceinline__ void bwd_weight(float s, float lse2, const BwdParams& p, float& w, float& dfac) {
+  if (p.softcap > 0.f) {
+    const float ex = __builtin_amdgcn_exp2f(s * p.cap_c2);
+    const float t = __builtin_fmaf(__builtin_amdgcn_rcpf(ex + 1.f), -2.f, 1.f);
+    w = __builtin_amdgcn_exp2f(__builtin_fmaf(t, p.softcap * 1.4426950408889634f, -lse2));
+    dfac = __builtin_fmaf(-t, t, 1.f);
+  } else {
+    w = __builtin_amdgcn_exp2f(__builtin_fmaf(s, p.sl2, -lse2));
+    dfac = 1.f;
+  }
+}
 
 template <int QB>
 struct BwdStep {
@@ -310,10 +327,13 @@ __global__ void __launch_bounds__(QB * 2, 1) bwd_dq_kernel(const BwdParams p) {
         constexpr int t = i / 8, r = 2 * (i % 8);
         constexpr int kl0 = 8 * (r >> 2) + (r & 3), kl1 = 8 * ((r + 1) >> 2) + ((r + 1) & 3);
         const bool keep0 = (kw[t] >> kl0) & 1u, keep1 = (kw[t] >> kl1) & 1u;
-        const float p0 = keep0 ? __builtin_amdgcn_exp2f(__builtin_fmaf(st[t][r], p.sl2, -lse2)) : 0.f;
-        const float p1 = keep1 ? __builtin_amdgcn_exp2f(__builtin_fmaf(st[t][r + 1], p.sl2, -lse2)) : 0.f;
-        const float d0 = p0 * (dp[t][r] - delta);
-        const float d1 = p1 * (dp[t][r + 1] - delta);
+        float w0, w1, f0, f1;
+        bwd_weight(st[t][r], lse2, p, w0, f0);
+        bwd_weight(st[t][r + 1], lse2, p, w1, f1);
+        const float p0 = keep0 ? w0 : 0.f;
+        const float p1 = keep1 ? w1 : 0.f;
+        const float d0 = p0 * (dp[t][r] - delta) * f0;
+        const float d1 = p1 * (dp[t][r + 1] - delta) * f1;
         dsb[t][r >> 3][(r & 7) >> 1] = pack2<BF16>(d0, d1);
       });
       // dQ^T += K^T.dS^T
@@ -495,9 +515,10 @@ __global__ void __launch_bounds__(KB * 2, 1) bwd_dkdv_kernel(const BwdParams p) 
               }
               keep = keep && bit;
             }
-            const float x = __builtin_fmaf(sc[t][4 * i4 + e], p.sl2, -l4[e]);
-            pv[e] = keep ? __builtin_amdgcn_exp2f(x) : 0.f;
-            dsv[e] = pv[e] * (dp[t][4 * i4 + e] - d4[e]);
+            float wgt, fac;
+            bwd_weight(sc[t][4 * i4 + e], l4[e], p, wgt, fac);
+            pv[e] = keep ? wgt : 0.f;
+            dsv[e] = pv[e] * (dp[t][4 * i4 + e] - d4[e]) * fac;
           }
           pb[t][i4 >> 1][2 * (i4 & 1) + 0] = pack2<BF16>(pv[0], pv[1]);
           pb[t][i4 >> 1][2 * (i4 & 1) + 1] = pack2<BF16>(pv[2], pv[3]);

@@ -78,7 +78,8 @@ int forward(const void* q, const void* k, const void* v, void* o, float* lse_or_
             const int32_t* kv_num_blocks, const int32_t* kv_indices, const int32_t* block_mask_types,
             const int32_t* partial_idx_or_null, const uint8_t* partial_masks_or_null,
             const uint32_t* partial_bits_or_null, int B, int H, int S_pad, int D, int Tq,
-            int max_blocks, int QB, int KB, int num_partial, int seqlen_orig, int dtype, void* stream) {
+            int max_blocks, int QB, int KB, int num_partial, int seqlen_orig, int dtype, float softcap,
+            void* stream) {
   using namespace omni_attn;
   if (!q || !k || !v || !o || !kv_num_blocks || !kv_indices || !block_mask_types)
     return OMNI_ATTN_ERR_NULL_POINTER;
@@ -95,6 +96,7 @@ int forward(const void* q, const void* k, const void* v, void* o, float* lse_or_
   if ((QB != 64 && QB != 128) || (KB != 64 && KB != 128)) return OMNI_ATTN_ERR_UNSUPPORTED_BLOCK;
   if (B <= 0 || H <= 0 || S_pad <= 0 || Tq <= 0 || max_blocks <= 0 || seqlen_orig < 0 || num_partial < 0)
     return OMNI_ATTN_ERR_BAD_SHAPE;
+  if (!(softcap >= 0.f) || std::isinf(softcap)) return OMNI_ATTN_ERR_BAD_SHAPE;  // also refuses NaN
   if (Tq != (S_pad + QB - 1) / QB) return OMNI_ATTN_ERR_BAD_SHAPE;
   const long long total = (long long)B * H * Tq;
   if ((long long)S_pad * D > 0x7fffffffLL || total > 0x7fffffffLL / 2 ||
@@ -149,7 +151,9 @@ int forward(const void* q, const void* k, const void* v, void* o, float* lse_or_
     while ((H / X) % heads != 0) --heads;  // whole batch elements per group sequence
   }
   p.slab_group = heads * ((fill + heads - 1) / heads);
-  p.sl2 = float(1.4426950408889634 / std::sqrt(double(D)));
+  p.softcap = softcap;
+  p.cap_c2 = softcap > 0.f ? float(2.0 * 1.4426950408889634 / (std::sqrt(double(D)) * double(softcap))) : 0.f;
+  p.sl2 = softcap > 0.f ? float(1.4426950408889634) : float(1.4426950408889634 / std::sqrt(double(D)));
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool bf = dtype == OMNI_ATTN_DTYPE_BF16;
@@ -173,10 +177,10 @@ extern "C" int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v,
                                     const int32_t* partial_idx_or_null,
                                     const uint8_t* partial_masks_or_null, int B, int H, int S_pad,
                                     int D, int Tq, int max_blocks, int QB, int KB, int num_partial,
-                                    int seqlen_orig, int dtype, void* stream) {
+                                    int seqlen_orig, int dtype, float softcap, void* stream) {
   return forward(q, k, v, o, lse_or_null, kv_num_blocks, kv_indices, block_mask_types, partial_idx_or_null,
                  partial_masks_or_null, nullptr, B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial,
-                 seqlen_orig, dtype, stream);
+                 seqlen_orig, dtype, softcap, stream);
 }
 
 extern "C" int omni_attn_fwd_packed_gfx950(const void* q, const void* k, const void* v, void* o,
@@ -185,10 +189,10 @@ extern "C" int omni_attn_fwd_packed_gfx950(const void* q, const void* k, const v
                                            const int32_t* partial_idx_or_null,
                                            const uint32_t* partial_bits_or_null, int B, int H, int S_pad,
                                            int D, int Tq, int max_blocks, int QB, int KB, int num_partial,
-                                           int seqlen_orig, int dtype, void* stream) {
+                                           int seqlen_orig, int dtype, float softcap, void* stream) {
   return forward(q, k, v, o, lse_or_null, kv_num_blocks, kv_indices, block_mask_types, partial_idx_or_null,
                  nullptr, partial_bits_or_null, B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial,
-                 seqlen_orig, dtype, stream);
+                 seqlen_orig, dtype, softcap, stream);
 }
 
 extern "C" size_t omni_attn_bwd_workspace_bytes(int B, int H, int S_pad) {
@@ -204,8 +208,9 @@ int backward(const void* q, const void* k, const void* v, const void* o, const v
              const int32_t* partial_idx_or_null, const uint8_t* partial_masks_or_null,
              const uint32_t* partial_bits_or_null, float* delta_workspace, int B, int H, int S_pad,
              int D, int Tq, int max_blocks, int QB, int KB, int num_partial, int seqlen_orig, int dtype,
-             void* stream) {
+             float softcap, void* stream) {
   using namespace omni_attn;
+  if (!(softcap >= 0.f) || std::isinf(softcap)) return OMNI_ATTN_ERR_BAD_SHAPE;
   if (!q || !k || !v || !o || !dout || !lse || !dq || !dk || !dv || !kv_num_blocks || !kv_indices ||
       !block_mask_types || !delta_workspace)
     return OMNI_ATTN_ERR_NULL_POINTER;
@@ -259,6 +264,8 @@ int backward(const void* q, const void* k, const void* v, const void* o, const v
   p.n_slabs = B * H;
   p.scale = float(1.0 / std::sqrt(double(D)));
   p.sl2 = float(1.4426950408889634 / std::sqrt(double(D)));
+  p.softcap = softcap;
+  p.cap_c2 = softcap > 0.f ? float(2.0 * 1.4426950408889634 / (std::sqrt(double(D)) * double(softcap))) : 0.f;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool bf = dtype == OMNI_ATTN_DTYPE_BF16;
@@ -284,13 +291,13 @@ extern "C" int omni_attn_bwd_gfx950(const void* q, const void* k, const void* v,
                                     const uint32_t* partial_bits_or_null, void* workspace,
                                     size_t workspace_bytes, int B, int H, int S_pad, int D, int Tq,
                                     int max_blocks, int QB, int KB, int num_partial, int seqlen_orig,
-                                    int dtype, void* stream) {
+                                    int dtype, float softcap, void* stream) {
   if (B > 0 && H > 0 && S_pad > 0 && workspace_bytes < omni_attn_bwd_workspace_bytes(B, H, S_pad))
     return OMNI_ATTN_ERR_WORKSPACE;
   return backward(q, k, v, o, dout, lse, dq, dk, dv, kv_num_blocks, kv_indices, block_mask_types,
                   partial_idx_or_null, partial_masks_or_null, partial_bits_or_null,
                   static_cast<float*>(workspace), B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial,
-                  seqlen_orig, dtype, stream);
+                  seqlen_orig, dtype, softcap, stream);
 }
 
 // ---- the backward for callers that cannot allocate -------------------------------------------
@@ -333,7 +340,7 @@ extern "C" int omni_attn_bwd_noalloc_gfx950(const void* q, const void* k, const 
                                             const uint8_t* partial_masks_or_null,
                                             const uint32_t* partial_bits_or_null, int B, int H, int S_pad,
                                             int D, int Tq, int max_blocks, int QB, int KB, int num_partial,
-                                            int seqlen_orig, int dtype, void* stream) {
+                                            int seqlen_orig, int dtype, float softcap, void* stream) {
   if (B <= 0 || H <= 0 || S_pad <= 0) return OMNI_ATTN_ERR_BAD_SHAPE;
   if ((unsigned long long)B * (unsigned long long)H * (unsigned long long)S_pad > kScratchFloats)
     return OMNI_ATTN_ERR_SCRATCH_LIMIT;
@@ -346,7 +353,7 @@ extern "C" int omni_attn_bwd_noalloc_gfx950(const void* q, const void* k, const 
   // slab before the dK/dV kernel, which runs after it on the same stream, reads any of them.
   return backward(q, k, v, o, dout, lse, dq, dk, dv, kv_num_blocks, kv_indices, block_mask_types,
                   partial_idx_or_null, partial_masks_or_null, partial_bits_or_null, delta, B, H, S_pad, D,
-                  Tq, max_blocks, QB, KB, num_partial, seqlen_orig, dtype, stream);
+                  Tq, max_blocks, QB, KB, num_partial, seqlen_orig, dtype, softcap, stream);
 }
 
 extern "C" const char* omni_attn_status_string(int status) {
@@ -370,4 +377,4 @@ extern "C" const char* omni_attn_status_string(int status) {
 
 extern "C" int omni_attn_last_hip_error(void) { return g_last_hip_error; }
 
-extern "C" int omni_attn_abi_version(void) { return 2; }
+extern "C" int omni_attn_abi_version(void) { return 3; }

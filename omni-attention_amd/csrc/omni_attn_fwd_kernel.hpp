@@ -74,7 +74,9 @@ struct FwdParams {
   int n_slabs;     // B*H
   int n_xcd;       // XCDs (L2 domains) of the device; workgroup ids go round-robin over them
   int slab_group;  // slabs of one XCD that are walked together (>= 1)
-  float sl2;       // log2(e) / sqrt(D)
+  float sl2;       // log2(e) / sqrt(D); log2(e) when scores are soft-capped (they are scaled there)
+  float softcap;   // > 0: scores s / sqrt(D) are replaced by softcap * tanh(s / sqrt(D) / softcap)
+  float cap_c2;    // 2 * log2(e) / (sqrt(D) * softcap)
 };
 
 template <bool BF16>
@@ -553,6 +555,22 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     });
   };
 
+  // Soft-capped scores (the score_mod of transfusion_pytorch/transfusion.py:358-364, applied to the
+  // scaled score as at :958-959 and :968): cap * tanh(x / cap) = cap * (1 - 2 / (exp(2 x / cap) + 1)),
+  // written into S^T before the mask and the softmax of the step; the softmax then runs on
+  // scores that are already scaled (sl2 = log2 e).
+  auto apply_softcap = [&](auto set_c) {
+    constexpr int SET = decltype(set_c)::value;
+    const float cap = p.softcap, c2 = p.cap_c2;
+    static_for<16 * NTL>([&](auto ec) {
+      constexpr int e = decltype(ec)::value;
+      constexpr int t = e / 16, r = e % 16;
+      const float ex = __builtin_amdgcn_exp2f(st[SET][t][r] * c2);
+      const float rc = __builtin_amdgcn_rcpf(ex + 1.f);
+      st[SET][t][r] = __builtin_fmaf(rc, -2.f * cap, cap);
+    });
+  };
+
   auto body = [&](auto set_c, auto first_c, int k_row0, int v_row0) {
     constexpr int SET = decltype(set_c)::value;
     // The first iteration of a walk has no previous step: no PV slots.
@@ -678,6 +696,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
         for (int r = 0; r < 16; ++r) ot[dt][r] *= alpha_pending;
       rescale_pending = 0;
     }
+    if (p.softcap > 0.f) apply_softcap(IntC<SET>{});
     if (!unmasked(cur)) apply_mask(IntC<SET>{}, cur);
     const bool next_partial = it + 1 < nsteps && nxt.mode == kPartial;
     if (next_partial) {

@@ -41,7 +41,8 @@ void forward_impl(const torch::Tensor& Q, const torch::Tensor& K, const torch::T
                   const torch::Tensor& kv_indices, const torch::Tensor& block_mask_types,
                   int Q_BLOCK_SIZE, int KV_BLOCK_SIZE, int seqlen_orig,
                   const torch::Tensor& partial_block_mask_indices,
-                  const torch::Tensor& partial_block_masks, bool has_partial, bool packed = false) {
+                  const torch::Tensor& partial_block_masks, bool has_partial, bool packed = false,
+                  double softcap = 0.0) {
   if (Q.scalar_type() != torch::kHalf && Q.scalar_type() != torch::kBFloat16)
     throw std::runtime_error("Tensor dtype mismatch: Q must be torch.float16 or torch.bfloat16");
   check_qkvo(Q, "Q", Q);
@@ -118,13 +119,13 @@ void forward_impl(const torch::Tensor& Q, const torch::Tensor& K, const torch::T
                    kv_num_blocks.data_ptr<int32_t>(), kv_indices.data_ptr<int32_t>(),
                    block_mask_types.data_ptr<int32_t>(), pidx, reinterpret_cast<const uint32_t*>(pmask),
                    int(B), int(H), int(S), int(D), int(num_q_blocks), int(max_blocks), Q_BLOCK_SIZE,
-                   KV_BLOCK_SIZE, num_partial, seqlen_orig, dtype, static_cast<void*>(stream))
+                   KV_BLOCK_SIZE, num_partial, seqlen_orig, dtype, float(softcap), static_cast<void*>(stream))
              : omni_attn_fwd_gfx950(
                    Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), lse,
                    kv_num_blocks.data_ptr<int32_t>(), kv_indices.data_ptr<int32_t>(),
                    block_mask_types.data_ptr<int32_t>(), pidx, pmask, int(B), int(H), int(S), int(D),
                    int(num_q_blocks), int(max_blocks), Q_BLOCK_SIZE, KV_BLOCK_SIZE, num_partial,
-                   seqlen_orig, dtype, static_cast<void*>(stream));
+                   seqlen_orig, dtype, float(softcap), static_cast<void*>(stream));
   if (rc != OMNI_ATTN_OK) {
     std::string msg = std::string("omni_attn: ") + omni_attn_status_string(rc);
     if (rc == OMNI_ATTN_ERR_UNSUPPORTED_HEAD_DIM) msg += ", got head_dim=" + std::to_string(D);
@@ -153,7 +154,7 @@ void omni_attn_forward(torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch:
                        torch::Tensor LSE, torch::Tensor kv_num_blocks, torch::Tensor kv_indices,
                        torch::Tensor block_mask_types, int Q_BLOCK_SIZE, int KV_BLOCK_SIZE,
                        int seqlen_orig, torch::Tensor partial_block_mask_indices,
-                       torch::Tensor partial_block_masks, bool has_partial) {
+                       torch::Tensor partial_block_masks, bool has_partial, double softcap) {
   if (LSE.scalar_type() != torch::kFloat32)
     throw std::runtime_error("Tensor dtype mismatch: LSE must be torch.float32");
   if (!LSE.is_contiguous() || LSE.dim() != 3 || Q.dim() != 4 || LSE.size(0) != Q.size(0) ||
@@ -161,7 +162,7 @@ void omni_attn_forward(torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch:
     throw std::runtime_error("LSE must be a contiguous [B, H, S] tensor on the device of Q");
   forward_impl(Q, K, V, O, LSE.data_ptr<float>(), kv_num_blocks, kv_indices, block_mask_types,
                Q_BLOCK_SIZE, KV_BLOCK_SIZE, seqlen_orig, partial_block_mask_indices,
-               partial_block_masks, has_partial);
+               partial_block_masks, has_partial, false, softcap);
 }
 
 // PARTIAL tiles [P, QB, KB] bool -> [P, QB, KB / 32] int32 words, packed on the GPU.
@@ -186,7 +187,7 @@ void omni_attn_forward_packed(torch::Tensor Q, torch::Tensor K, torch::Tensor V,
                               torch::Tensor LSE, torch::Tensor kv_num_blocks, torch::Tensor kv_indices,
                               torch::Tensor block_mask_types, int Q_BLOCK_SIZE, int KV_BLOCK_SIZE,
                               int seqlen_orig, torch::Tensor partial_block_mask_indices,
-                              torch::Tensor partial_block_bits) {
+                              torch::Tensor partial_block_bits, double softcap) {
   float* lse = nullptr;
   if (LSE.numel() > 0) {
     if (LSE.scalar_type() != torch::kFloat32)
@@ -197,7 +198,7 @@ void omni_attn_forward_packed(torch::Tensor Q, torch::Tensor K, torch::Tensor V,
     lse = LSE.data_ptr<float>();
   }
   forward_impl(Q, K, V, O, lse, kv_num_blocks, kv_indices, block_mask_types, Q_BLOCK_SIZE, KV_BLOCK_SIZE,
-               seqlen_orig, partial_block_mask_indices, partial_block_bits, true, true);
+               seqlen_orig, partial_block_mask_indices, partial_block_bits, true, true, softcap);
 }
 
 // Backward of omni_attn_forward: dQ, dK, dV written in place (the reference exports no backward).
@@ -207,7 +208,7 @@ void omni_attn_backward(torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch
                         torch::Tensor dV, torch::Tensor kv_num_blocks, torch::Tensor kv_indices,
                         torch::Tensor block_mask_types, int Q_BLOCK_SIZE, int KV_BLOCK_SIZE,
                         int seqlen_orig, torch::Tensor partial_block_mask_indices,
-                        torch::Tensor partial_tiles, bool has_partial, bool packed) {
+                        torch::Tensor partial_tiles, bool has_partial, bool packed, double softcap) {
   if (Q.scalar_type() != torch::kHalf && Q.scalar_type() != torch::kBFloat16)
     throw std::runtime_error("Tensor dtype mismatch: Q must be torch.float16 or torch.bfloat16");
   check_qkvo(Q, "Q", Q);
@@ -261,7 +262,7 @@ void omni_attn_backward(torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch
       kv_indices.data_ptr<int32_t>(), block_mask_types.data_ptr<int32_t>(), pidx,
       packed ? nullptr : static_cast<const uint8_t*>(tiles), packed ? static_cast<const uint32_t*>(tiles) : nullptr,
       workspace.data_ptr(), ws_bytes, int(B), int(H), int(S), int(D), int(kv_num_blocks.size(2)),
-      int(kv_indices.size(3)), Q_BLOCK_SIZE, KV_BLOCK_SIZE, num_partial, seqlen_orig, dtype,
+      int(kv_indices.size(3)), Q_BLOCK_SIZE, KV_BLOCK_SIZE, num_partial, seqlen_orig, dtype, float(softcap),
       static_cast<void*>(stream));
   if (rc != OMNI_ATTN_OK) {
     std::string msg = std::string("omni_attn: ") + omni_attn_status_string(rc);
@@ -282,11 +283,24 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("omni_attn_preftech", &omni_attn_op, "omni_attn_preftech");
   m.def("omni_attn_mma_stages_split_q_shared_kv_swizzle", &omni_attn_op,
         "omni_attn_mma_stages_split_q_shared_kv_swizzle");
-  m.def("omni_attn_forward", &omni_attn_forward, "omni_attn_forward (also writes logsumexp)");
+  namespace py = pybind11;
+  m.def("omni_attn_forward", &omni_attn_forward, "omni_attn_forward (also writes logsumexp)", py::arg("Q"),
+        py::arg("K"), py::arg("V"), py::arg("O"), py::arg("LSE"), py::arg("kv_num_blocks"), py::arg("kv_indices"),
+        py::arg("block_mask_types"), py::arg("Q_BLOCK_SIZE"), py::arg("KV_BLOCK_SIZE"), py::arg("seqlen_orig"),
+        py::arg("partial_block_mask_indices"), py::arg("partial_block_masks"), py::arg("has_partial"),
+        py::arg("softcap") = 0.0);
   m.def("omni_attn_pack_partial_masks", &omni_attn_pack_partial_masks,
         "omni_attn_pack_partial_masks (bool tiles -> 32-bit words)");
   m.def("omni_attn_forward_packed", &omni_attn_forward_packed,
-        "omni_attn_forward_packed (PARTIAL tiles as packed words)");
-  m.def("omni_attn_backward", &omni_attn_backward, "omni_attn_backward (dQ, dK, dV of omni_attn_forward)");
+        "omni_attn_forward_packed (PARTIAL tiles as packed words)", py::arg("Q"), py::arg("K"), py::arg("V"),
+        py::arg("O"), py::arg("LSE"), py::arg("kv_num_blocks"), py::arg("kv_indices"), py::arg("block_mask_types"),
+        py::arg("Q_BLOCK_SIZE"), py::arg("KV_BLOCK_SIZE"), py::arg("seqlen_orig"),
+        py::arg("partial_block_mask_indices"), py::arg("partial_block_bits"), py::arg("softcap") = 0.0);
+  m.def("omni_attn_backward", &omni_attn_backward, "omni_attn_backward (dQ, dK, dV of omni_attn_forward)",
+        py::arg("Q"), py::arg("K"), py::arg("V"), py::arg("O"), py::arg("dO"), py::arg("LSE"), py::arg("dQ"),
+        py::arg("dK"), py::arg("dV"), py::arg("kv_num_blocks"), py::arg("kv_indices"), py::arg("block_mask_types"),
+        py::arg("Q_BLOCK_SIZE"), py::arg("KV_BLOCK_SIZE"), py::arg("seqlen_orig"),
+        py::arg("partial_block_mask_indices"), py::arg("partial_tiles"), py::arg("has_partial"), py::arg("packed"),
+        py::arg("softcap") = 0.0);
   m.def("abi_version", []() { return omni_attn_abi_version(); });
 }

@@ -40,18 +40,18 @@ def load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(LIB_PATH)
         vp, i32 = ctypes.c_void_p, ctypes.c_int
         lib.omni_attn_fwd_gfx950.restype = i32
-        lib.omni_attn_fwd_gfx950.argtypes = [vp] * 10 + [i32] * 11 + [vp]
+        lib.omni_attn_fwd_gfx950.argtypes = [vp] * 10 + [i32] * 11 + [ctypes.c_float, vp]
         lib.omni_attn_fwd_packed_gfx950.restype = i32
-        lib.omni_attn_fwd_packed_gfx950.argtypes = [vp] * 10 + [i32] * 11 + [vp]
+        lib.omni_attn_fwd_packed_gfx950.argtypes = [vp] * 10 + [i32] * 11 + [ctypes.c_float, vp]
         lib.omni_attn_pack_partial_masks_gfx950.restype = i32
         lib.omni_attn_pack_partial_masks_gfx950.argtypes = [vp, vp, i32, i32, i32, vp]
         lib.omni_attn_bwd_workspace_bytes.restype = ctypes.c_size_t
         lib.omni_attn_bwd_workspace_bytes.argtypes = [i32, i32, i32]
         lib.omni_attn_bwd_gfx950.restype = i32
-        lib.omni_attn_bwd_gfx950.argtypes = [vp] * 16 + [ctypes.c_size_t] + [i32] * 11 + [vp]
+        lib.omni_attn_bwd_gfx950.argtypes = [vp] * 16 + [ctypes.c_size_t] + [i32] * 11 + [ctypes.c_float, vp]
         lib.omni_attn_bwd_noalloc_max_rows.restype = ctypes.c_size_t
         lib.omni_attn_bwd_noalloc_gfx950.restype = i32
-        lib.omni_attn_bwd_noalloc_gfx950.argtypes = [vp] * 15 + [i32] * 11 + [vp]
+        lib.omni_attn_bwd_noalloc_gfx950.argtypes = [vp] * 15 + [i32] * 11 + [ctypes.c_float, vp]
         lib.omni_attn_mfma_peak_probe_gfx950.restype = i32
         lib.omni_attn_mfma_peak_probe_gfx950.argtypes = [i32, i32, vp, ctypes.POINTER(ctypes.c_double), vp]
         lib.omni_attn_status_string.restype = ctypes.c_char_p
@@ -83,11 +83,12 @@ def _ptr(t: Optional[torch.Tensor]) -> int:
 
 
 def fwd_raw(q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, nb_ptr, idx_ptr, types_ptr, pidx_ptr, pmask_ptr,
-            B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial, seqlen_orig, dtype, stream_ptr) -> int:
+            B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial, seqlen_orig, dtype, stream_ptr,
+            softcap: float = 0.0) -> int:
     """The C call itself; returns the status code."""
     return load_library().omni_attn_fwd_gfx950(
         q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, nb_ptr, idx_ptr, types_ptr, pidx_ptr, pmask_ptr,
-        B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial, seqlen_orig, dtype, stream_ptr)
+        B, H, S_pad, D, Tq, max_blocks, QB, KB, num_partial, seqlen_orig, dtype, softcap, stream_ptr)
 
 
 def pack_partial_masks(partial_masks: torch.Tensor, stream: Optional[int] = None) -> torch.Tensor:
@@ -108,7 +109,8 @@ def pack_partial_masks(partial_masks: torch.Tensor, stream: Optional[int] = None
 
 
 def fwd(q, k, v, o, lse, kv_num_blocks, kv_indices, block_mask_types, QB, KB, seqlen_orig,
-        partial_idx=None, partial_masks=None, stream: Optional[int] = None, partial_bits=None) -> None:
+        partial_idx=None, partial_masks=None, stream: Optional[int] = None, partial_bits=None,
+        softcap: float = 0.0) -> None:
     """Enqueue the forward on ``stream`` (default: torch's current stream of q's device).
     q, k, v, o: contiguous [B, H, S_pad, D] fp16 or bf16 on the GPU; lse: fp32 [B, H, S_pad]
     or None.  PARTIAL tiles either as bytes (``partial_masks``) or packed by
@@ -146,7 +148,8 @@ def fwd(q, k, v, o, lse, kv_num_blocks, kv_indices, block_mask_types, QB, KB, se
                 _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(kv_num_blocks), _ptr(kv_indices),
                 _ptr(block_mask_types), _ptr(partial_idx if partial_bits.shape[0] else None),
                 _ptr(partial_bits if partial_bits.shape[0] else None), B, H, S, D, kv_num_blocks.shape[2],
-                kv_indices.shape[3], QB, KB, int(partial_bits.shape[0]), int(seqlen_orig), dtype, stream)
+                kv_indices.shape[3], QB, KB, int(partial_bits.shape[0]), int(seqlen_orig), dtype, float(softcap),
+                stream)
         if rc != 0:
             raise RuntimeError("omni_attn_fwd_packed_gfx950: %s (status %d)" % (status_string(rc), rc))
         return
@@ -155,14 +158,14 @@ def fwd(q, k, v, o, lse, kv_num_blocks, kv_indices, block_mask_types, QB, KB, se
                      _ptr(kv_indices), _ptr(block_mask_types), _ptr(partial_idx), _ptr(partial_masks),
                      B, H, S, D, kv_num_blocks.shape[2], kv_indices.shape[3], QB, KB,
                      0 if partial_masks is None else int(partial_masks.shape[0]),
-                     int(seqlen_orig), dtype, stream)
+                     int(seqlen_orig), dtype, stream, float(softcap))
     if rc != 0:
         raise RuntimeError("omni_attn_fwd_gfx950: %s (status %d)" % (status_string(rc), rc))
 
 
 def bwd(q, k, v, o, dout, lse, dq, dk, dv, kv_num_blocks, kv_indices, block_mask_types, QB, KB, seqlen_orig,
         partial_idx=None, partial_masks=None, partial_bits=None, workspace: Optional[torch.Tensor] = None,
-        stream: Optional[int] = None, no_alloc: bool = False) -> None:
+        stream: Optional[int] = None, no_alloc: bool = False, softcap: float = 0.0) -> None:
     """Enqueue the backward (two kernels) on ``stream``.  All of q, k, v, o, dout, dq, dk, dv are
     contiguous [B, H, S_pad, D] GPU tensors of one 16-bit dtype, lse is the forward's fp32
     [B, H, S_pad].  ``workspace``: a GPU tensor of at least omni_attn_bwd_workspace_bytes bytes
@@ -203,7 +206,7 @@ def bwd(q, k, v, o, dout, lse, dq, dk, dv, kv_num_blocks, kv_indices, block_mask
                 _ptr(kv_num_blocks), _ptr(kv_indices), _ptr(block_mask_types), _ptr(partial_idx),
                 _ptr(partial_masks if partial_bits is None else None), _ptr(partial_bits),
                 B, H, S, D, kv_num_blocks.shape[2], kv_indices.shape[3], QB, KB, num_partial, int(seqlen_orig),
-                dtype, stream)
+                dtype, float(softcap), stream)
         if rc != 0:
             raise RuntimeError("omni_attn_bwd_noalloc_gfx950: %s (status %d)" % (status_string(rc), rc))
         return
@@ -213,6 +216,6 @@ def bwd(q, k, v, o, dout, lse, dq, dk, dv, kv_num_blocks, kv_indices, block_mask
             _ptr(kv_num_blocks), _ptr(kv_indices), _ptr(block_mask_types), _ptr(partial_idx),
             _ptr(partial_masks if partial_bits is None else None), _ptr(partial_bits), _ptr(workspace), ws_bytes,
             B, H, S, D, kv_num_blocks.shape[2], kv_indices.shape[3], QB, KB, num_partial, int(seqlen_orig),
-            dtype, stream)
+            dtype, float(softcap), stream)
     if rc != 0:
         raise RuntimeError("omni_attn_bwd_gfx950: %s (status %d)" % (status_string(rc), rc))

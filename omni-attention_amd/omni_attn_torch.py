@@ -482,7 +482,7 @@ _SUPPORTED_BLOCKS = (64, 128)
 
 def _omni_attention(op_name: str, query: Tensor, key: Tensor, value: Tensor,
                     block_mask: OmniBlockMask, partial_needs_partial_types: bool,
-                    return_lse: bool = False, keep_padded: bool = False):
+                    return_lse: bool = False, keep_padded: bool = False, softcap: float = 0.0):
     ext = _load_extension()
     B, H, Q, D = query.shape
     KV = key.shape[2]
@@ -551,23 +551,25 @@ def _omni_attention(op_name: str, query: Tensor, key: Tensor, value: Tensor,
 
     if has_partial and block_mask.partial_block_bits is not None and block_mask.partial_block_bits.device == dev:
         # tiles packed once by OmniBlockMask.pack_partial_masks(): same kernel, packed input
-        lse_padded = (torch.empty(B, H, S_pad, dtype=torch.float32, device=dev) if return_lse
+        lse_padded = (torch.empty(B, H, S_pad, dtype=torch.float32, device=dev) if (return_lse or keep_padded)
                       else torch.empty(0, dtype=torch.float32, device=dev))
         ext.omni_attn_forward_packed(query_padded, key_padded, value_padded, output_padded, lse_padded,
                                      kv_num_blocks, kv_indices, block_mask_types, QB, KB, q_orig_len,
-                                     partial_idx, block_mask.partial_block_bits.contiguous())
+                                     partial_idx, block_mask.partial_block_bits.contiguous(), float(softcap))
         if keep_padded:
             return output_padded, lse_padded, query_padded, key_padded, value_padded, q_orig_len
         if return_lse:
             return output_padded[:, :, :q_orig_len, :], lse_padded[:, :, :q_orig_len]
         return output_padded[:, :, :q_orig_len, :]
-    if return_lse:
+    if return_lse or softcap:
         lse_padded = torch.empty(B, H, S_pad, dtype=torch.float32, device=dev)
         ext.omni_attn_forward(query_padded, key_padded, value_padded, output_padded, lse_padded,
                               kv_num_blocks, kv_indices, block_mask_types, QB, KB, q_orig_len,
-                              partial_idx, partial_masks, has_partial)
+                              partial_idx, partial_masks, has_partial, float(softcap))
         if keep_padded:
             return output_padded, lse_padded, query_padded, key_padded, value_padded, q_orig_len
+        if not return_lse:
+            return output_padded[:, :, :q_orig_len, :]
         return output_padded[:, :, :q_orig_len, :], lse_padded[:, :, :q_orig_len]
     getattr(ext, op_name)(query_padded, key_padded, value_padded, output_padded,
                           kv_num_blocks, kv_indices, block_mask_types, QB, KB, q_orig_len,
@@ -607,10 +609,11 @@ def omni_attention_shared_kv_swizzle(query: Tensor, key: Tensor, value: Tensor,
 
 
 def omni_attention_forward(query: Tensor, key: Tensor, value: Tensor,
-                           block_mask: OmniBlockMask) -> Tuple[Tensor, Tensor]:
+                           block_mask: OmniBlockMask, softcap: float = 0.0) -> Tuple[Tensor, Tensor]:
     """Output and fp32 row logsumexp [B, H, S] (-inf for rows with no allowed key).
     Not in the reference, which has no logsumexp output."""
-    return _omni_attention("omni_attn_forward", query, key, value, block_mask, False, return_lse=True)
+    return _omni_attention("omni_attn_forward", query, key, value, block_mask, False, return_lse=True,
+                           softcap=softcap)
 
 
 class _OmniAttentionFunction(torch.autograd.Function):
@@ -620,12 +623,14 @@ class _OmniAttentionFunction(torch.autograd.Function):
     transfusion_pytorch/transfusion.py:953-983."""
 
     @staticmethod
-    def forward(ctx, query, key, value, block_mask):
+    def forward(ctx, query, key, value, block_mask, softcap):
         out_padded, lse_padded, q_pad, k_pad, v_pad, seq_len = _omni_attention(
-            "omni_attn_forward", query, key, value, block_mask, False, return_lse=True, keep_padded=True)
+            "omni_attn_forward", query, key, value, block_mask, False, return_lse=True, keep_padded=True,
+            softcap=softcap)
         ctx.save_for_backward(q_pad, k_pad, v_pad, out_padded, lse_padded)
         ctx.block_mask = block_mask
         ctx.seq_len = seq_len
+        ctx.softcap = float(softcap)
         return out_padded[:, :, :seq_len, :]
 
     @staticmethod
@@ -652,14 +657,18 @@ class _OmniAttentionFunction(torch.autograd.Function):
             tiles = torch.empty(0, dtype=torch.bool, device=dev)
         ext.omni_attn_backward(q_pad, k_pad, v_pad, out_padded, d_out, lse_padded, dq, dk, dv,
                                to_i32(m.kv_num_blocks), to_i32(m.kv_indices), to_i32(m.block_mask_types),
-                               m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, seq_len, pidx, tiles, has_partial, packed)
-        return dq[:, :, :seq_len, :], dk[:, :, :seq_len, :], dv[:, :, :seq_len, :], None
+                               m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, seq_len, pidx, tiles, has_partial, packed,
+                               ctx.softcap)
+        return dq[:, :, :seq_len, :], dk[:, :, :seq_len, :], dv[:, :, :seq_len, :], None, None
 
 
-def omni_attention(query: Tensor, key: Tensor, value: Tensor, block_mask: OmniBlockMask) -> Tensor:
+def omni_attention(query: Tensor, key: Tensor, value: Tensor, block_mask: OmniBlockMask,
+                   softcap: float = 0.0) -> Tensor:
     """Differentiable block-sparse attention: the forward kernel, with the backward kernels
-    behind ``.backward()`` (gradients with respect to query, key and value)."""
-    return _OmniAttentionFunction.apply(query, key, value, block_mask)
+    behind ``.backward()`` (gradients with respect to query, key and value).  ``softcap`` > 0
+    replaces the scaled score x by softcap * tanh(x / softcap) before mask and softmax
+    (transfusion_pytorch/transfusion.py:358-364)."""
+    return _OmniAttentionFunction.apply(query, key, value, block_mask, float(softcap))
 
 
 # ----------------------------------------------------------------------------

@@ -13,9 +13,13 @@ import torch
 
 
 def attention_dense_fp32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
-                         mask: torch.Tensor, row_chunk: int = 2048) -> Tuple[torch.Tensor, torch.Tensor]:
+                         mask: torch.Tensor, row_chunk: int = 2048,
+                         softcap: float = 0.0) -> Tuple[torch.Tensor, torch.Tensor]:
     """q, k, v: [..., S, D] (any float dtype, converted to fp32 as they are);
     mask: bool, broadcastable to [..., S, S], True = attend.
+    softcap > 0: scaled scores x become softcap * tanh(x / softcap) before the mask, the way
+    Transfusion's attention layer does it (transfusion_pytorch/transfusion.py:298-299 softclamp,
+    :358-364 the flex score_mod, :966-968 the dense path).
     Returns (O fp32 [..., S, D], LSE fp32 [..., S])."""
     qf, kf, vf = q.float(), k.float(), v.float()
     S, D = qf.shape[-2], qf.shape[-1]
@@ -25,6 +29,8 @@ def attention_dense_fp32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     for r0 in range(0, S, row_chunk):
         r1 = min(S, r0 + row_chunk)
         s = torch.matmul(qf[..., r0:r1, :], kf.transpose(-1, -2)) * scale
+        if softcap > 0:
+            s = torch.tanh(s / softcap) * softcap
         m = mask[..., r0:r1, :]
         s = s.masked_fill(~m, float("-inf"))
         any_row = m.any(-1)
@@ -38,12 +44,14 @@ def attention_dense_fp32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
 
 
 def attention_dense_differentiable(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
-                                   mask: torch.Tensor) -> torch.Tensor:
+                                   mask: torch.Tensor, softcap: float = 0.0) -> torch.Tensor:
     """The same function as attention_dense_fp32 (output only) written so that autograd can
     go through it, in the dtype of its inputs (fp32, or fp64 for gradcheck): rows with no
     allowed key give 0 and pass no gradient."""
     D = q.shape[-1]
     s = torch.matmul(q, k.transpose(-1, -2)) / math.sqrt(D)
+    if softcap > 0:
+        s = torch.tanh(s / softcap) * softcap
     any_row = mask.any(-1, keepdim=True)
     s = s.masked_fill(~mask, float("-inf"))
     s = torch.where(any_row, s, torch.zeros_like(s))  # keeps softmax finite on empty rows
@@ -53,11 +61,11 @@ def attention_dense_differentiable(q: torch.Tensor, k: torch.Tensor, v: torch.Te
 
 
 def attention_dense_grads(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor,
-                          dout: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+                          dout: torch.Tensor, softcap: float = 0.0) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """(dQ, dK, dV) of sum(O * dout) by autograd through attention_dense_differentiable in fp32
     (inputs of any float dtype are converted as they are)."""
     qf, kf, vf = (t.detach().float().clone().requires_grad_(True) for t in (q, k, v))
-    out = attention_dense_differentiable(qf, kf, vf, mask)
+    out = attention_dense_differentiable(qf, kf, vf, mask, softcap)
     out.backward(dout.float())
     return qf.grad, kf.grad, vf.grad
 

@@ -28,26 +28,28 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(omni_attn_capi.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert omni_attn_capi.load_library().omni_attn_abi_version() == 2
+    assert omni_attn_capi.load_library().omni_attn_abi_version() == 3
 
 
 def test_argument_validation_codes():
     lib = omni_attn_capi.load_library()
     one = 4096  # any non-null value: validation fails before it would be dereferenced
-    def call(q=one, D=128, QB=128, KB=128, Tq=4, S=512, dtype=1, B=1, P=0):
+    def call(q=one, D=128, QB=128, KB=128, Tq=4, S=512, dtype=1, B=1, P=0, softcap=0.0):
         return omni_attn_capi.fwd_raw(q, one, one, one, 0, one, one, one, 0, 0,
-                                      B, 2, S, D, Tq, 4, QB, KB, P, S, dtype, 0)
+                                      B, 2, S, D, Tq, 4, QB, KB, P, S, dtype, 0, softcap)
     assert call(q=0) == 1
     assert call(B=0) == 2
     assert call(Tq=5) == 2            # Tq != ceil(S / QB)
     assert call(P=-1) == 2            # negative number of stored partial tiles
+    assert call(softcap=-1.0) == 2    # softcap must be 0 (off) or positive and finite
+    assert call(softcap=float("nan")) == 2 and call(softcap=float("inf")) == 2
     assert call(D=96) == 3
     assert call(D=256) == 3
     assert call(QB=32) == 4
     assert call(KB=256) == 4
     assert call(dtype=7) == 5
     assert call(q=one + 8) == 8     # 16-byte alignment of q, k, v, o
-    for code in range(0, 9):
+    for code in range(0, 11):
         assert omni_attn_capi.status_string(code)
     assert "head_dim" in omni_attn_capi.status_string(3)
 
@@ -58,7 +60,7 @@ def test_python_module_surface():
                  "omni_attn_preftech_kernel", "omni_attn_preftech",
                  "omni_attn_mma_stages_split_q_shared_kv_swizzle", "omni_attn_forward"):
         assert callable(getattr(omni_attn, name)), name
-    assert omni_attn.abi_version() == 2
+    assert omni_attn.abi_version() == 3
     assert os.path.dirname(omni_attn.__file__) == PKG
 
 

@@ -47,5 +47,5 @@ def test_no_alloc_backward_rejects_sizes_beyond_its_scratch(gpu_device):
     assert max_rows == 4 << 20
     one = 4096  # non-null: the size check comes before any pointer is used
     rc = lib.omni_attn_bwd_noalloc_gfx950(one, one, one, one, one, one, one, one, one, one, one, one, 0, 0, 0,
-                                          64, 64, 2048, 128, 16, 16, 128, 128, 0, 2048, 1, 0)
+                                          64, 64, 2048, 128, 16, 16, 128, 128, 0, 2048, 1, 0.0, 0)
     assert rc == 10 and "scratch" in omni_attn_capi.status_string(rc)
