@@ -115,6 +115,25 @@ int omni_attn_fwd_gfx950(const void* q, const void* k, const void* v, void* o,
                          int seqlen_orig, int dtype, float softcap, void* stream);
 
 /*
+ * The same operation for shapes the MFMA kernel has no instance for: any QB > 0, KB > 0 and any
+ * D in 1..256 -- the generality of the reference's scalar kernel omni_attn_simple_kernel
+ * (omni-attn-mma/mma/attn_naive.cu:21-302; D <= 256 from its `float out[256]`, :189-190; its
+ * launcher :305-408 has no block-size or head-dim whitelist).  Same arguments, semantics and
+ * status codes as omni_attn_fwd_gfx950 (pointers need only their natural alignment); two-pass
+ * fp32 softmax per query row like the reference's kernel.  A correctness path, not a fast one.
+ */
+int omni_attn_fwd_generic_gfx950(const void* q, const void* k, const void* v, void* o,
+                                 float* lse_or_null,
+                                 const int32_t* kv_num_blocks,
+                                 const int32_t* kv_indices,
+                                 const int32_t* block_mask_types,
+                                 const int32_t* partial_idx_or_null,
+                                 const uint8_t* partial_masks_or_null,
+                                 int B, int H, int S_pad, int D,
+                                 int Tq, int max_blocks, int QB, int KB, int num_partial,
+                                 int seqlen_orig, int dtype, float softcap, void* stream);
+
+/*
  * Pre-pass for masks that are reused over many launches: packs the bool tiles that the
  * reference's build_partial_block_data produces (omni-attn-mma/omni_attn_torch.py:148-205,
  * [P, QB, KB] bytes) into [P, QB, KB / 32] 32-bit words, bit j of word c of a row = key

@@ -49,7 +49,7 @@ RESOURCES_JSON = os.path.join(OBJ, "kernel_resources.json")
 # The backward kernels are the plain schedule (one wave per SIMD, registers spilling into the
 # accumulation file, a few instances into scratch): they are recorded, not gated.
 MIN_WAVES_PER_SIMD = {"fwd_kernel": 2}
-NOT_GATED = ("bwd_dq_kernel", "bwd_dkdv_kernel")
+NOT_GATED = ("bwd_dq_kernel", "bwd_dkdv_kernel", "fwd_generic_kernel")
 
 INSTANCES = [(bf, d) for bf in (0, 1) for d in (32, 64, 128)]
 LIB_NAME = "libomni_attn_gfx950.so"
@@ -133,7 +133,7 @@ def build_capi(jobs):
         cmds.append([HIPCC] + DEVICE_FLAGS + [
             "-DOMNI_INST_BF16=%d" % bf, "-DOMNI_INST_D=%d" % d,
             "-c", os.path.join(CSRC, "omni_attn_bwd_inst.hip"), "-o", obj])
-    for src in ("omni_attn_capi", "omni_attn_probe", "omni_attn_mask_pack"):
+    for src in ("omni_attn_capi", "omni_attn_probe", "omni_attn_mask_pack", "omni_attn_fwd_generic"):
         obj = os.path.join(OBJ, src + ".o")
         objs.append(obj)
         cmds.append([HIPCC] + DEVICE_FLAGS + ["-c", os.path.join(CSRC, src + ".hip"), "-o", obj])

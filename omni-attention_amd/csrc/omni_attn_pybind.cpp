@@ -42,7 +42,7 @@ void forward_impl(const torch::Tensor& Q, const torch::Tensor& K, const torch::T
                   int Q_BLOCK_SIZE, int KV_BLOCK_SIZE, int seqlen_orig,
                   const torch::Tensor& partial_block_mask_indices,
                   const torch::Tensor& partial_block_masks, bool has_partial, bool packed = false,
-                  double softcap = 0.0) {
+                  double softcap = 0.0, bool generic_fallback = false) {
   if (Q.scalar_type() != torch::kHalf && Q.scalar_type() != torch::kBFloat16)
     throw std::runtime_error("Tensor dtype mismatch: Q must be torch.float16 or torch.bfloat16");
   check_qkvo(Q, "Q", Q);
@@ -113,8 +113,20 @@ void forward_impl(const torch::Tensor& Q, const torch::Tensor& K, const torch::T
   c10::DeviceGuard guard(Q.device());
   hipStream_t stream = c10::hip::getCurrentHIPStream(Q.device().index()).stream();
   const int dtype = Q.scalar_type() == torch::kBFloat16 ? OMNI_ATTN_DTYPE_BF16 : OMNI_ATTN_DTYPE_F16;
+  // The scalar entry point of the reference takes any block size and any head_dim <= 256
+  // (omni-attn-mma/mma/attn_naive.cu:189-190, :305-408): shapes without an MFMA instance go to
+  // the generic kernel when the caller is that entry point.
+  const bool has_instance = (D == 32 || D == 64 || D == 128) && (Q_BLOCK_SIZE == 64 || Q_BLOCK_SIZE == 128) &&
+                            (KV_BLOCK_SIZE == 64 || KV_BLOCK_SIZE == 128);
   const int rc =
-      packed ? omni_attn_fwd_packed_gfx950(
+      (generic_fallback && !has_instance && !packed)
+          ? omni_attn_fwd_generic_gfx950(
+                Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), lse,
+                kv_num_blocks.data_ptr<int32_t>(), kv_indices.data_ptr<int32_t>(),
+                block_mask_types.data_ptr<int32_t>(), pidx, pmask, int(B), int(H), int(S), int(D),
+                int(num_q_blocks), int(max_blocks), Q_BLOCK_SIZE, KV_BLOCK_SIZE, num_partial, seqlen_orig,
+                dtype, float(softcap), static_cast<void*>(stream))
+      : packed ? omni_attn_fwd_packed_gfx950(
                    Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), lse,
                    kv_num_blocks.data_ptr<int32_t>(), kv_indices.data_ptr<int32_t>(),
                    block_mask_types.data_ptr<int32_t>(), pidx, reinterpret_cast<const uint32_t*>(pmask),
@@ -147,6 +159,18 @@ void omni_attn_op(torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch::Tens
   forward_impl(Q, K, V, O, nullptr, kv_num_blocks, kv_indices, block_mask_types, Q_BLOCK_SIZE,
                KV_BLOCK_SIZE, seqlen_orig, partial_block_mask_indices, partial_block_masks,
                has_partial);
+}
+
+// omni_attn_simple_kernel: as above, and like the reference's scalar kernel for any Q_BLOCK_SIZE,
+// KV_BLOCK_SIZE and head_dim <= 256.
+void omni_attn_simple_op(torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch::Tensor O,
+                         torch::Tensor kv_num_blocks, torch::Tensor kv_indices,
+                         torch::Tensor block_mask_types, int Q_BLOCK_SIZE, int KV_BLOCK_SIZE,
+                         int seqlen_orig, torch::Tensor partial_block_mask_indices,
+                         torch::Tensor partial_block_masks, bool has_partial) {
+  forward_impl(Q, K, V, O, nullptr, kv_num_blocks, kv_indices, block_mask_types, Q_BLOCK_SIZE,
+               KV_BLOCK_SIZE, seqlen_orig, partial_block_mask_indices, partial_block_masks,
+               has_partial, false, 0.0, true);
 }
 
 // Same arguments plus LSE [B, H, S] fp32, written in place.
@@ -277,7 +301,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "gfx950 block-sparse FlashAttention-2 forward (omni-attention operator surface)";
   m.def("omni_attn_mma_stages_split_q_shared_kv", &omni_attn_op,
         "omni_attn_mma_stages_split_q_shared_kv");
-  m.def("omni_attn_simple_kernel", &omni_attn_op, "omni_attn_simple_kernel");
+  m.def("omni_attn_simple_kernel", &omni_attn_simple_op, "omni_attn_simple_kernel");
   m.def("omni_attn_cp_async", &omni_attn_op, "omni_attn_cp_async");
   m.def("omni_attn_preftech_kernel", &omni_attn_op, "omni_attn_preftech_kernel");
   m.def("omni_attn_preftech", &omni_attn_op, "omni_attn_preftech");

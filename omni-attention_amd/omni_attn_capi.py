@@ -20,6 +20,7 @@ DTYPE_BF16 = 1
 EXPORTED_SYMBOLS = (
     "omni_attn_fwd_gfx950",
     "omni_attn_fwd_packed_gfx950",
+    "omni_attn_fwd_generic_gfx950",
     "omni_attn_pack_partial_masks_gfx950",
     "omni_attn_bwd_gfx950",
     "omni_attn_bwd_workspace_bytes",
@@ -41,6 +42,8 @@ def load_library() -> ctypes.CDLL:
         vp, i32 = ctypes.c_void_p, ctypes.c_int
         lib.omni_attn_fwd_gfx950.restype = i32
         lib.omni_attn_fwd_gfx950.argtypes = [vp] * 10 + [i32] * 11 + [ctypes.c_float, vp]
+        lib.omni_attn_fwd_generic_gfx950.restype = i32
+        lib.omni_attn_fwd_generic_gfx950.argtypes = [vp] * 10 + [i32] * 11 + [ctypes.c_float, vp]
         lib.omni_attn_fwd_packed_gfx950.restype = i32
         lib.omni_attn_fwd_packed_gfx950.argtypes = [vp] * 10 + [i32] * 11 + [ctypes.c_float, vp]
         lib.omni_attn_pack_partial_masks_gfx950.restype = i32
@@ -110,7 +113,7 @@ def pack_partial_masks(partial_masks: torch.Tensor, stream: Optional[int] = None
 
 def fwd(q, k, v, o, lse, kv_num_blocks, kv_indices, block_mask_types, QB, KB, seqlen_orig,
         partial_idx=None, partial_masks=None, stream: Optional[int] = None, partial_bits=None,
-        softcap: float = 0.0) -> None:
+        softcap: float = 0.0, generic: bool = False) -> None:
     """Enqueue the forward on ``stream`` (default: torch's current stream of q's device).
     q, k, v, o: contiguous [B, H, S_pad, D] fp16 or bf16 on the GPU; lse: fp32 [B, H, S_pad]
     or None.  PARTIAL tiles either as bytes (``partial_masks``) or packed by
@@ -152,6 +155,16 @@ def fwd(q, k, v, o, lse, kv_num_blocks, kv_indices, block_mask_types, QB, KB, se
                 stream)
         if rc != 0:
             raise RuntimeError("omni_attn_fwd_packed_gfx950: %s (status %d)" % (status_string(rc), rc))
+        return
+    if generic:
+        with torch.cuda.device(q.device):
+            rc = load_library().omni_attn_fwd_generic_gfx950(
+                _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(kv_num_blocks), _ptr(kv_indices),
+                _ptr(block_mask_types), _ptr(partial_idx), _ptr(partial_masks), B, H, S, D, kv_num_blocks.shape[2],
+                kv_indices.shape[3], QB, KB, 0 if partial_masks is None else int(partial_masks.shape[0]),
+                int(seqlen_orig), dtype, float(softcap), stream)
+        if rc != 0:
+            raise RuntimeError("omni_attn_fwd_generic_gfx950: %s (status %d)" % (status_string(rc), rc))
         return
     with torch.cuda.device(q.device):
         rc = fwd_raw(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(kv_num_blocks),

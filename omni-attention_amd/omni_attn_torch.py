@@ -521,12 +521,18 @@ def _omni_attention(op_name: str, query: Tensor, key: Tensor, value: Tensor,
             f"q_len ({block_mask.q_len}) must be a multiple of KV_BLOCK_SIZE ({KB}) so that Q, K and V "
             f"share one padded length")
 
-    if D not in _SUPPORTED_HEAD_DIMS:
-        raise ValueError(f"Unsupported head_dim={D}. Supported values: 32, 64, 128.")
-    if QB not in _SUPPORTED_BLOCKS:
-        raise ValueError(f"Unsupported Q_BLOCK_SIZE={QB}. Supported values: 64, 128.")
-    if KB not in _SUPPORTED_BLOCKS:
-        raise ValueError(f"Unsupported KV_BLOCK_SIZE={KB}. Supported values: 64, 128.")
+    # the scalar entry point takes any block size and head_dim <= 256, like the reference's
+    # (attn_naive.cu:189-190, :305-408); the others only the shapes with an MFMA instance
+    if op_name == "omni_attn_simple_kernel":
+        if not 0 < D <= 256:
+            raise ValueError(f"Unsupported head_dim={D}. Supported values: 1..256.")
+    else:
+        if D not in _SUPPORTED_HEAD_DIMS:
+            raise ValueError(f"Unsupported head_dim={D}. Supported values: 32, 64, 128.")
+        if QB not in _SUPPORTED_BLOCKS:
+            raise ValueError(f"Unsupported Q_BLOCK_SIZE={QB}. Supported values: 64, 128.")
+        if KB not in _SUPPORTED_BLOCKS:
+            raise ValueError(f"Unsupported KV_BLOCK_SIZE={KB}. Supported values: 64, 128.")
 
     dev = query.device
     query_padded = query_padded.contiguous()
