@@ -210,6 +210,87 @@ def band_sweep(dev, steps, warmup):
     }
 
 
+def fixed_cost_study(dev, seed, steps, warmup):
+    """Where the time of c2_interleaved goes besides the per-block work: the same launch with
+    every list repeated 2x and 3x (same workgroups, 2x / 3x the steps: r*T1 - Tr is r - 1 times the
+    part that does not grow with the lists), with all block types FULL (no mask work), with the
+    same number of blocks spread evenly over the query blocks (no imbalance), and the dense and
+    plain causal controls of the same shape.  Kernel times are medians of HIP-event brackets."""
+    import torch
+
+    import omni_attn_capi
+    from baseline_configs import make_workload
+
+    w = make_workload("c2_interleaved", seed=seed)
+    m = w.block_mask
+    B, H, S, D = w.q.shape
+    QB, KB = m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE
+    q, k, v = (t.to(dev) for t in (w.q, w.k, w.v))
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, S, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    per_block = 4.0 * QB * KB * D
+    nb0, idx0, tys0 = m.kv_num_blocks, m.kv_indices, m.block_mask_types
+    Tq, MB = nb0.shape[2], idx0.shape[3]
+
+    def run(nb, idx, tys, what):
+        nbd, idxd, tysd = (t.to(dev).contiguous() for t in (nb, idx, tys))
+
+        def step():
+            omni_attn_capi.fwd(q, k, v, o, lse, nbd, idxd, tysd, QB, KB, S, None, None, stream=stream.cuda_stream)
+
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        st = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        en = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        for i in range(steps):
+            st[i].record(stream)
+            step()
+            en[i].record(stream)
+        torch.cuda.synchronize()
+        ms = statistics.median(a.elapsed_time(b) for a, b in zip(st, en))
+        blocks = int(nb.sum().item())
+        return {"case": what, "listed_blocks": blocks, "kernel_us": ms * 1e3,
+                "tflops": per_block * blocks / (ms * 1e-3) / 1e12, "ns_per_block": ms * 1e6 / blocks}
+
+    t_end = time.perf_counter() + 0.25  # settle the clock under this load
+    nbd, idxd, tysd = (t.to(dev) for t in (nb0, idx0, tys0))
+    while time.perf_counter() < t_end:
+        for _ in range(10):
+            omni_attn_capi.fwd(q, k, v, o, lse, nbd, idxd, tysd, QB, KB, S, None, None, stream=stream.cuda_stream)
+        torch.cuda.synchronize()
+    rows = [run(nb0, idx0, tys0, "c2_interleaved as it is")]
+    T1 = rows[0]["kernel_us"]
+    ar = torch.arange(MB * 3)
+    for r in (2, 3):
+        idx = torch.zeros(B, H, Tq, MB * r, dtype=torch.int32)
+        tys = torch.zeros(B, H, Tq, MB * r, dtype=torch.int32)
+        for b in range(B):
+            src = (ar[: MB * r].view(1, -1) % nb0[b, 0].clamp(min=1).view(-1, 1)).long()
+            idx[b] = torch.gather(idx0[b, 0], 1, src).unsqueeze(0).expand(H, -1, -1)
+            tys[b] = torch.gather(tys0[b, 0], 1, src).unsqueeze(0).expand(H, -1, -1)
+        row = run(nb0 * r, idx, tys, f"every list repeated {r}x")
+        row["fixed_us_estimate"] = (r * T1 - row["kernel_us"]) / (r - 1)
+        rows.append(row)
+    rows.append(run(nb0, idx0, torch.where(tys0 == 1, torch.full_like(tys0, 2), tys0), "all listed blocks FULL"))
+    tot = int(nb0.sum().item())
+    per = tot // (B * H * Tq)
+    nbb = torch.full((B, H, Tq), per, dtype=torch.int32)
+    nbb.view(-1)[: tot - per * B * H * Tq] += 1
+    idxb = torch.arange(MB, dtype=torch.int32).expand(B, H, Tq, MB).contiguous()
+    tysb = torch.full((B, H, Tq, MB), 2, dtype=torch.int32)
+    rows.append(run(nbb, idxb, tysb, "same total, spread evenly over the query blocks"))
+    rows.append(run(torch.full((B, H, Tq), MB, dtype=torch.int32), idxb, tysb, "dense control"))
+    nbc = (torch.arange(Tq, dtype=torch.int32) + 1).expand(B, H, Tq).contiguous()
+    tysc = tysb.clone()
+    for i in range(Tq):
+        tysc[:, :, i, i] = 1
+    rows.append(run(nbc, idxb, tysc, "plain causal"))
+    return {"study": "c2_interleaved: fixed cost, mask cost, imbalance (B=2 H=32 S=4096 D=128 bf16, 128/128)",
+            "rows": rows}
+
+
 def extra_workload(name, seed, dev, steps, warmup):
     """Kernel time of another workload (HIP events on the launch stream, clock already settled)."""
     import torch
@@ -272,6 +353,9 @@ def main(argv=None):
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, so that a counter run of this "
                          "command shows what FETCH_SIZE / WRITE_SIZE read for a known traffic")
+    ap.add_argument("--fixed-cost", action="store_true",
+                    help="instead of the workload: c2_interleaved with its lists repeated, its types all "
+                         "FULL, its blocks spread evenly (fixed cost / mask cost / imbalance of a launch)")
     ap.add_argument("--sweep-bands", action="store_true",
                     help="instead of the workload: kernel time against the number of listed blocks")
     args = ap.parse_args(argv)
@@ -296,6 +380,9 @@ def main(argv=None):
     omni_attn_capi.load_library()  # fail loudly when the HIP library is missing
     if args.sweep_bands:
         print(json.dumps(band_sweep(dev, min(args.steps, 30), min(args.warmup, 5))))
+        return 0
+    if args.fixed_cost:
+        print(json.dumps(fixed_cost_study(dev, args.seed, min(args.steps, 60), min(args.warmup, 10))))
         return 0
 
     w = make_workload(args.workload, seed=args.seed)
