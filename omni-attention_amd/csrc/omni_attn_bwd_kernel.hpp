@@ -17,6 +17,8 @@
 //   bwd_dkdv_kernel  one workgroup per KV block; finds the (query block, slot) pairs that list
 //                    it by scanning the slab's metadata (a bitmap of the matches is built in
 //                    LDS first, then visited in ascending order).
+// The dQ kernel runs two workgroups per compute unit (two waves per SIMD, each hides the other's
+// loads); the dK/dV kernel needs more than 256 registers per lane and runs one.
 // Both use the forward's building blocks with the operands exchanged: every product is a
 // v_mfma_f32_32x32x16 whose A operand comes from an LDS tile (row-wise or transposed read)
 // and whose B operand is in registers, and the accumulator of the first product of a step is
@@ -180,7 +182,7 @@ struct BwdDqTraits {
 };
 
 template <bool BF16, int D, int QB, int KB>
-__global__ void __launch_bounds__(QB * 2, 1) bwd_dq_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   using Traits = BwdDqTraits<D, QB>;
   constexpr int NT = Traits::kThreads;
   constexpr int STEP = Traits::kStep;
@@ -351,7 +353,9 @@ __global__ void __launch_bounds__(QB * 2, 1) bwd_dq_kernel(const BwdParams p) {
 template <int D, int KB>
 struct BwdDkdvTraits {
   static constexpr int kThreads = KB * 2;
-  static constexpr int kStep = BwdStep<KB>::value;  // query rows per step
+  // query rows per step: 32 where the tile still divides over the workgroup (two accumulator
+  // pairs per wave already fill most of the register file), else the forward's rule
+  static constexpr int kStep = (32 * (D / 8) % (KB * 2) == 0) ? 32 : BwdStep<KB>::value;
   static constexpr int kTileElems = kStep * D;
   static constexpr int kMaxBitmapWords = 4096;      // 64-slot words of the match bitmap (32 KiB)
   // four tiles (Q and dO, each row-wise and transposed) or the output staging, + lse and delta of a
