@@ -199,7 +199,7 @@ int omni_attn_bwd_gfx950(const void* q, const void* k, const void* v, const void
  * omni_attn_bwd_gfx950 for callers that cannot allocate device memory for the workspace: code
  * under HIP graph capture, tight serving or training loops, harnesses that forbid allocation.
  * No counterpart in the reference.  Same kernels and bit-identical results; the workspace is a
- * 16 MiB device array built into the library (each GPU the library runs on holds its copy until
+ * 32 MiB device array built into the library (each GPU the library runs on holds its copy until
  * the process ends), so B * H * S_pad must not exceed omni_attn_bwd_noalloc_max_rows()
  * (4 194 304), else OMNI_ATTN_ERR_SCRATCH_LIMIT.  Calls no hipMalloc / hipFree or any other
  * allocating routine.  All calls on one GPU share that GPU's array: calls that overlap in time

@@ -23,7 +23,8 @@
 // v_mfma_f32_32x32x16 whose A operand comes from an LDS tile (row-wise or transposed read)
 // and whose B operand is in registers, and the accumulator of the first product of a step is
 // the B operand of the second one, so P and dS never leave registers.
-// Tiles are single-buffered: this is the straightforward schedule, not the forward's pipeline.
+// Tiles are double-buffered (the loads of step i + 1 run under the products of step i, one barrier
+// per step); inside a step the products and the vector work are left to the compiler's schedule.
 #pragma once
 
 #include "omni_attn_fwd_kernel.hpp"
@@ -42,7 +43,10 @@ struct BwdParams {
   uint16_t* dq;
   uint16_t* dk;
   uint16_t* dv;
-  float* delta;  // [B,H,S] workspace: written by the dQ kernel, read by the dK/dV kernel
+  // workspace [2][B,H,S], written by the dQ kernel and read by the dK/dV kernel: plane 0 is
+  // -delta = -rowsum(dO . O); plane 1 the exponent offset of the row, LSE * log2(e), +inf for a
+  // row without any allowed key or beyond the sequence (every weight of such a row becomes 0)
+  float* ws;
   const int32_t* kv_num_blocks;
   const int32_t* kv_indices;
   const int32_t* types;
@@ -60,8 +64,9 @@ struct BwdParams {
 // Weight and score-gradient factor of one score.  Plain: p = exp2(s * sl2 - lse2), factor 1.
 // Soft-capped: t = tanh(s / sqrt(D) / cap), p = exp2(cap * t * log2 e - lse2), factor 1 - t^2
 // (the derivative of cap * tanh(x / cap) with respect to x).
+template <bool CAP>
 __device__ __forceinline__ void bwd_weight(float s, float lse2, const BwdParams& p, float& w, float& dfac) {
-  if (p.softcap > 0.f) {
+  if constexpr (CAP) {
     const float ex = __builtin_amdgcn_exp2f(s * p.cap_c2);
     const float t = __builtin_fmaf(__builtin_amdgcn_rcpf(ex + 1.f), -2.f, 1.f);
     w = __builtin_amdgcn_exp2f(__builtin_fmaf(t, p.softcap * 1.4426950408889634f, -lse2));
@@ -70,6 +75,39 @@ __device__ __forceinline__ void bwd_weight(float s, float lse2, const BwdParams&
     w = __builtin_amdgcn_exp2f(__builtin_fmaf(s, p.sl2, -lse2));
     dfac = 1.f;
   }
+}
+
+// LDS reads at a byte address.  A fragment's address is (tile + lane part) ^ (k-step bits) + a
+// constant: the swizzles of both tile layouts only touch the chunk bits inside a row, and they
+// repeat every 16 rows, so rows and tiles are immediate offsets and a fragment costs one XOR.
+__device__ __forceinline__ u32x4_t lds_b128_at(uint32_t addr) {
+  return *(const __attribute__((address_space(3))) u32x4_t*)(addr);
+}
+__device__ __forceinline__ f32x4_t lds_f32x4_at(uint32_t addr) {
+  return *(const __attribute__((address_space(3))) f32x4_t*)(addr);
+}
+__device__ __forceinline__ u32x4_t lds_tr_pair_at(uint32_t addr, uint32_t hi_off) {
+  const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(addr));
+  const s16x4_t hi =
+      __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(addr + hi_off));
+  const u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo);
+  const u32x2_t hi2 = __builtin_bit_cast(u32x2_t, hi);
+  const u32x4_t a = {lo2[0], lo2[1], hi2[0], hi2[1]};
+  return a;
+}
+// Lane part (bytes) of a row-wise A fragment: row 32 t + c of the tile, k-step s at
+// ((tile + lane part) ^ 32 s) + 32 t rows.
+template <int D>
+__device__ __forceinline__ uint32_t bwd_row_lane(int g, int c) {
+  return uint32_t(c * D + (g ^ k_swizzle<D>(c)) * 8) * 2u;
+}
+// Lane part (bytes) of a transposed A fragment: rows 32 dt .. +31 of tile^T at tile rows
+// 16 ts .. +15 (taken in the accumulator order of the first product) at
+// ((tile + lane part) ^ 64 dt) + 16 ts rows, second half 8 rows further.
+template <int D>
+__device__ __forceinline__ uint32_t bwd_tr_lane(int g, int c) {
+  const int i16 = c & 15, j16 = c >> 4, r0 = 4 * g + (i16 >> 2);
+  return uint32_t(r0 * D + (j16 ^ v_swizzle<D>(r0)) * 16 + (i16 & 3) * 4) * 2u;
 }
 
 template <int QB>
@@ -83,9 +121,11 @@ struct BwdStep {
 template <int D, int NT, int ROWS, bool TR>
 __device__ __forceinline__ void bwd_load_tile(i32x4_t rsrc, int row0, uint32_t lds_tile, int tid, int w) {
   constexpr int CPR = D / 8;
-  constexpr int NCH = ROWS * CPR / NT;
-  static_assert(ROWS * CPR % NT == 0 && NCH >= 1, "tile must divide over the workgroup");
+  constexpr int TOTAL = ROWS * CPR;  // 16-byte chunks of the tile
+  constexpr int NCH = TOTAL >= NT ? TOTAL / NT : 1;
+  static_assert(TOTAL >= NT ? TOTAL % NT == 0 : TOTAL % 64 == 0, "tile must divide over the threads (or whole waves)");
   constexpr int ROW_STRIDE = NT / CPR;
+  if (TOTAL < NT && tid >= TOTAL) return;  // a small tile is loaded by the first waves only
   const int ld_row = tid / CPR, ld_pch = tid % CPR;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
@@ -172,16 +212,33 @@ __device__ __forceinline__ void bwd_store_rows(const f32x16_t (&acc)[D / 32], fl
   }
 }
 
+// Rows of a backward tile: 32 where a [32][D] tile still divides over the workgroup (two sets
+// of tiles then leave room for two workgroups per compute unit), else 64.
+template <int D, int NT>
+struct BwdRows {
+  static constexpr int value = (32 * (D / 8) % NT == 0) ? 32 : 64;
+};
+
+// One step of a backward walk.
+struct BwdStepInfo {
+  int row0;   // first key row (dQ kernel) / first query row (dK/dV kernel) of the step
+  int mode;   // effective block mode
+  int pid;    // partial tile
+  int blk;    // dK/dV kernel: query block of the step
+  int sub;    // index of the step inside its block
+  bool valid;
+};
+
 template <int D, int QB>
 struct BwdDqTraits {
   static constexpr int kThreads = QB * 2;
-  static constexpr int kStep = BwdStep<QB>::value;
+  static constexpr int kStep = BwdRows<D, kThreads>::value;
   static constexpr int kTileElems = kStep * D;
-  // three tiles (K row-wise, K transposed, V row-wise) or the output staging, whichever is larger
-  static constexpr size_t kLdsBytes = (3 * kTileElems > QB * D ? 3 * kTileElems : QB * D) * sizeof(uint16_t);
+  // two sets of three tiles (K row-wise, K transposed, V row-wise), or the output staging
+  static constexpr size_t kLdsBytes = (6 * kTileElems > QB * D ? 6 * kTileElems : QB * D) * sizeof(uint16_t);
 };
 
-template <bool BF16, int D, int QB, int KB>
+template <bool BF16, bool CAP, int D, int QB, int KB>
 __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   using Traits = BwdDqTraits<D, QB>;
   constexpr int NT = Traits::kThreads;
@@ -193,9 +250,7 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   constexpr int TILE = Traits::kTileElems;
 
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-  uint16_t* sKa = reinterpret_cast<uint16_t*>(lds_raw);
-  uint16_t* sKt = sKa + TILE;
-  uint16_t* sVa = sKt + TILE;
+  uint16_t* const lds16 = reinterpret_cast<uint16_t*>(lds_raw);  // [2 sets][Ka, Kt, Va][TILE]
 
   const int bh = blockIdx.x / p.Tq;
   const int qb = p.Tq - 1 - (blockIdx.x - bh * p.Tq);
@@ -215,6 +270,19 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   const size_t meta_off = meta_row * p.max_blocks;
   const bool has_partial = p.partial_idx != nullptr && (p.partial_masks != nullptr || p.partial_bits != nullptr);
 
+  // Block metadata in registers, as in the forward: lane i holds block 64 * chunk + i of the list.
+  int32_t mv_kvb = 0, mv_mode = kMasked, mv_pid = -1;
+  auto load_chunk = [&](int chunk) {
+    const int j = chunk * 64 + lane;
+    const size_t o = meta_off + size_t(j < p.max_blocks ? j : 0);
+    const int32_t raw = p.kv_indices[o];
+    const int32_t ty = p.types[o];
+    const int32_t pid = has_partial ? p.partial_idx[o] : -1;
+    mv_kvb = raw < 0 ? 0 : (raw >= p.Tk ? p.Tk - 1 : raw);
+    mv_mode = bwd_slot_mode(ty, pid, has_partial, p.num_partial);
+    mv_pid = pid;
+  };
+  load_chunk(0);
   int nb = load_uniform(p.kv_num_blocks + meta_row);
   nb = nb < 0 ? 0 : (nb > p.max_blocks ? p.max_blocks : nb);
 
@@ -257,302 +325,526 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   const bool row_live = q_row < p.seqlen && lse != -INFINITY;
   // exponent offset; +inf for rows without any allowed key so that every weight becomes 0
   const float lse2 = row_live ? lse * 1.4426950408889634f : INFINITY;
-  if (q_row < p.S && g == 0) p.delta[size_t(bh) * p.S + q_row] = delta;
+  if (q_row < p.S && g == 0) {
+    p.ws[size_t(bh) * p.S + q_row] = -delta;
+    p.ws[size_t(p.n_slabs) * p.S + size_t(bh) * p.S + q_row] = lse2;
+  }
 
   const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   f32x16_t dq[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) dq[dt] = zero16;
 
-  for (int j = 0; j < nb; ++j) {
-    const size_t o = meta_off + size_t(j);
-    const int32_t kvb_raw = load_uniform(p.kv_indices + o);
-    const int32_t ty = load_uniform(p.types + o);
-    const int32_t pid = has_partial ? load_uniform(p.partial_idx + o) : -1;
-    const int32_t kvb = kvb_raw < 0 ? 0 : (kvb_raw >= p.Tk ? p.Tk - 1 : kvb_raw);
-    const int32_t mode = bwd_slot_mode(ty, pid, has_partial, p.num_partial);
-    if (mode == kMasked) continue;
-    for (int half = 0; half < SPB; ++half) {
-      const int row0 = kvb * KB + half * STEP;
-      if (row0 >= p.seqlen) continue;                                  // no allowed key
-      if (mode == kCausal && row0 > qb * QB + QB - 1) continue;        // entirely above the diagonal
-      __syncthreads();  // the previous step's operand reads are done
-      bwd_load_tile<D, NT, STEP, false>(rK, row0, lds_offset_of(sKa), tid, w);
-      bwd_load_tile<D, NT, STEP, true>(rK, row0, lds_offset_of(sKt), tid, w);
-      bwd_load_tile<D, NT, STEP, false>(rV, row0, lds_offset_of(sVa), tid, w);
-      // mask words of this lane's row: bit j of word t = key row0 + 32 t + j allowed
-      uint32_t kw[NTL];
+  // The steps of the walk in order, skipping what contributes nothing: MASKED slots, keys at or
+  // beyond the sequence, CAUSAL steps entirely above the diagonal of this query block.
+  int gj = 0, gsub = 0;
+  auto next_step = [&]() {
+    BwdStepInfo st = {0, kMasked, -1, 0, 0, false};
+    while (gj < nb) {
+      if (gsub == 0 && (gj & 63) == 0 && gj > 0) load_chunk(gj >> 6);
+      const int ln = gj & 63;
+      const int kvb = __builtin_amdgcn_readlane(mv_kvb, ln);
+      const int mode = __builtin_amdgcn_readlane(mv_mode, ln);
+      const int pid = __builtin_amdgcn_readlane(mv_pid, ln);
+      const int sub = gsub;
+      if (mode == kMasked || ++gsub == SPB) {
+        gsub = 0;
+        ++gj;
+      }
+      if (mode == kMasked) continue;
+      const int row0 = kvb * KB + sub * STEP;
+      if (row0 >= p.seqlen) continue;
+      if (mode == kCausal && row0 > qb * QB + QB - 1) continue;
+      st.row0 = row0;
+      st.mode = mode;
+      st.pid = pid;
+      st.sub = sub;
+      st.valid = true;
+      break;
+    }
+    return st;
+  };
+  const uint32_t lds_tiles = lds_offset_of(lds16);
+  auto issue_loads = [&](const BwdStepInfo& st, int set) {
+    const uint32_t base = lds_tiles + uint32_t(set) * (3u * TILE * 2u);
+    bwd_load_tile<D, NT, STEP, false>(rK, st.row0, base, tid, w);
+    bwd_load_tile<D, NT, STEP, true>(rK, st.row0, base + TILE * 2u, tid, w);
+    bwd_load_tile<D, NT, STEP, false>(rV, st.row0, base + 2u * TILE * 2u, tid, w);
+  };
+  const uint32_t row_lane = bwd_row_lane<D>(g, c);
+  const uint32_t tr_lane = bwd_tr_lane<D>(g, c);
+  constexpr int PF = KS < 3 ? KS : 3;  // k-steps whose fragments are read ahead of their products
+
+  // One step: S^T = K.Q^T and dP^T = V.dO^T (lane = query row, registers = keys), then
+  // dS^T = P^T (dP^T - delta) packed to 16 bits in the order the next product reads it, then
+  // dQ^T += K^T.dS^T.
+  auto compute = [&](int set, const uint32_t (&kw)[NTL]) {
+    const uint32_t base = lds_tiles + uint32_t(set) * (3u * TILE * 2u);
+    const uint32_t aK = base + row_lane, aV = aK + 2u * TILE * 2u, tK = base + TILE * 2u + tr_lane;
+    f32x16_t st[NTL], dp[NTL];
+    static_for<NTL>([&](auto tc) {
+      constexpr int t = decltype(tc)::value;
+      constexpr uint32_t trow = uint32_t(t) * 32u * D * 2u;
+      u32x4_t fa[KS], fb[KS];
+      static_for<PF>([&](auto sc) {
+        constexpr int s = decltype(sc)::value;
+        fa[s] = lds_b128_at((aK ^ uint32_t(32 * s)) + trow);
+        fb[s] = lds_b128_at((aV ^ uint32_t(32 * s)) + trow);
+      });
+      static_for<KS>([&](auto sc) {
+        constexpr int s = decltype(sc)::value;
+        if constexpr (s + PF < KS) {
+          fa[s + PF] = lds_b128_at((aK ^ uint32_t(32 * (s + PF))) + trow);
+          fb[s + PF] = lds_b128_at((aV ^ uint32_t(32 * (s + PF))) + trow);
+        }
+        st[t] = mfma_32x32x16<BF16>(fa[s], qf[s], s == 0 ? zero16 : st[t]);
+        dp[t] = mfma_32x32x16<BF16>(fb[s], dof[s], s == 0 ? zero16 : dp[t]);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
+    constexpr int NTS = STEP / 16;
+    u32x4_t ft[NTS][DT];  // fragments of the second product, read one 16-key group ahead
+    static_for<DT>([&](auto dc) {
+      constexpr int dt = decltype(dc)::value;
+      ft[0][dt] = lds_tr_pair_at(tK ^ uint32_t(64 * dt), 8u * D * 2u);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    u32x4_t dsb[NTL][2];
+    static_for<8 * NTL>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      constexpr int t = i / 8, r = 2 * (i % 8);
+      constexpr int kl0 = 8 * (r >> 2) + (r & 3), kl1 = 8 * ((r + 1) >> 2) + ((r + 1) & 3);
+      const bool keep0 = (kw[t] >> kl0) & 1u, keep1 = (kw[t] >> kl1) & 1u;
+      float w0, w1, f0, f1;
+      bwd_weight<CAP>(st[t][r], lse2, p, w0, f0);
+      bwd_weight<CAP>(st[t][r + 1], lse2, p, w1, f1);
+      const float p0 = keep0 ? w0 : 0.f;
+      const float p1 = keep1 ? w1 : 0.f;
+      const float d0 = p0 * (dp[t][r] - delta) * f0;
+      const float d1 = p1 * (dp[t][r + 1] - delta) * f1;
+      dsb[t][r >> 3][(r & 7) >> 1] = pack2<BF16>(d0, d1);
+    });
+    static_for<NTS>([&](auto tsc) {
+      constexpr int ts = decltype(tsc)::value;
+      if constexpr (ts + 1 < NTS) {
+        static_for<DT>([&](auto dc) {
+          constexpr int dt = decltype(dc)::value;
+          ft[ts + 1][dt] = lds_tr_pair_at((tK ^ uint32_t(64 * dt)) + uint32_t(ts + 1) * 16u * D * 2u, 8u * D * 2u);
+        });
+      }
+      static_for<DT>([&](auto dc) {
+        constexpr int dt = decltype(dc)::value;
+        dq[dt] = mfma_32x32x16<BF16>(ft[ts][dt], dsb[ts >> 1][ts & 1], dq[dt]);
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+
+  // Tiles of step i + 1 are loaded while step i is computed: one barrier per step.
+  BwdStepInfo cur = next_step();
+  int set = 0;
+  if (cur.valid) issue_loads(cur, 0);
+  while (cur.valid) {
+    const BwdStepInfo nxt = next_step();
+    // mask words of this lane's row: bit j of word t = key row0 + 32 t + j allowed
+    uint32_t kw[NTL];
 #pragma unroll
-      for (int t = 0; t < NTL; ++t) kw[t] = 0xffffffffu;
-      if (mode == kPartial) {
-        const int q_local = q_row - qb * QB;
+    for (int t = 0; t < NTL; ++t) kw[t] = 0xffffffffu;
+    if (cur.mode == kPartial) {
+      const int q_local = q_row - qb * QB;
 #pragma unroll
-        for (int t = 0; t < NTL; ++t) {
-          const int kcol = half * STEP + 32 * t;
-          if (p.partial_bits != nullptr) {
-            kw[t] = p.partial_bits[(size_t(pid) * QB + q_local) * (KB / 32) + kcol / 32];
-          } else {
-            const uint8_t* mp = p.partial_masks + (size_t(pid) * QB + q_local) * KB + kcol;
-            kw[t] = bwd_pack32(*reinterpret_cast<const u32x4_t*>(mp), *reinterpret_cast<const u32x4_t*>(mp + 16));
-          }
+      for (int t = 0; t < NTL; ++t) {
+        const int kcol = cur.sub * STEP + 32 * t;
+        if (p.partial_bits != nullptr) {
+          kw[t] = p.partial_bits[(size_t(cur.pid) * QB + q_local) * (KB / 32) + kcol / 32];
+        } else {
+          const uint8_t* mp = p.partial_masks + (size_t(cur.pid) * QB + q_local) * KB + kcol;
+          kw[t] = bwd_pack32(*reinterpret_cast<const u32x4_t*>(mp), *reinterpret_cast<const u32x4_t*>(mp + 16));
         }
       }
-      int limit = p.seqlen - 1;
-      if (mode == kCausal) limit = limit < q_row ? limit : q_row;
-      const int lim_l = limit - row0 - 4 * g;
-      static_for<NTL>([&](auto tc) {
-        constexpr int t = decltype(tc)::value;
-        kw[t] >>= 4 * g;
-        const int n = lim_l - 32 * t + 1;
-        const uint32_t low = n >= 32 ? 0xffffffffu : (n <= 0 ? 0u : ((1u << (n & 31)) - 1u));
-        kw[t] &= low;
-      });
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): tiles (and mask words) have landed
-      __syncthreads();
-
-      // S^T = K.Q^T and dP^T = V.dO^T : lane = query row, registers = keys
-      f32x16_t st[NTL], dp[NTL];
-      static_for<NTL>([&](auto tc) {
-        constexpr int t = decltype(tc)::value;
-        st[t] = zero16;
-        dp[t] = zero16;
-        static_for<KS>([&](auto sc) {
-          constexpr int s = decltype(sc)::value;
-          st[t] = mfma_32x32x16<BF16>(bwd_row_frag<D>(sKa, s, t, g, c), qf[s], st[t]);
-          dp[t] = mfma_32x32x16<BF16>(bwd_row_frag<D>(sVa, s, t, g, c), dof[s], dp[t]);
-        });
-      });
-      // dS^T = P^T (dP^T - delta), packed to 16 bits in the order the next product reads it
-      u32x4_t dsb[NTL][2];
-      static_for<8 * NTL>([&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        constexpr int t = i / 8, r = 2 * (i % 8);
-        constexpr int kl0 = 8 * (r >> 2) + (r & 3), kl1 = 8 * ((r + 1) >> 2) + ((r + 1) & 3);
-        const bool keep0 = (kw[t] >> kl0) & 1u, keep1 = (kw[t] >> kl1) & 1u;
-        float w0, w1, f0, f1;
-        bwd_weight(st[t][r], lse2, p, w0, f0);
-        bwd_weight(st[t][r + 1], lse2, p, w1, f1);
-        const float p0 = keep0 ? w0 : 0.f;
-        const float p1 = keep1 ? w1 : 0.f;
-        const float d0 = p0 * (dp[t][r] - delta) * f0;
-        const float d1 = p1 * (dp[t][r + 1] - delta) * f1;
-        dsb[t][r >> 3][(r & 7) >> 1] = pack2<BF16>(d0, d1);
-      });
-      // dQ^T += K^T.dS^T
-      static_for<(STEP / 16) * DT>([&](auto jc) {
-        constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
-        dq[dt] = mfma_32x32x16<BF16>(bwd_tr_frag<D>(sKt, ts, dt, g, c), dsb[ts >> 1][ts & 1], dq[dt]);
-      });
     }
+    int limit = p.seqlen - 1;
+    if (cur.mode == kCausal) limit = limit < q_row ? limit : q_row;
+    const int lim_l = limit - cur.row0 - 4 * g;
+    static_for<NTL>([&](auto tc) {
+      constexpr int t = decltype(tc)::value;
+      kw[t] >>= 4 * g;
+      const int n = lim_l - 32 * t + 1;
+      const uint32_t low = n >= 32 ? 0xffffffffu : (n <= 0 ? 0u : ((1u << (n & 31)) - 1u));
+      kw[t] &= low;
+    });
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this step's tiles (and mask words) have landed
+    __syncthreads();                     // ... for every wave; and the other set is no longer read
+    if (nxt.valid) issue_loads(nxt, set ^ 1);
+    compute(set, kw);
+    set ^= 1;
+    cur = nxt;
   }
   __syncthreads();  // tiles are dead: the staging area overlaps them
-  uint16_t* stage = reinterpret_cast<uint16_t*>(lds_raw) + size_t(w) * 32 * D;
+  uint16_t* stage = lds16 + size_t(w) * 32 * D;
   bwd_store_rows<BF16, D>(dq, p.scale, stage, p.dq + slab, q_wave_min, p.S, lane);
 }
 
 template <int D, int KB>
 struct BwdDkdvTraits {
-  static constexpr int kThreads = KB * 2;
-  // query rows per step: 32 where the tile still divides over the workgroup (two accumulator
-  // pairs per wave already fill most of the register file), else the forward's rule
-  static constexpr int kStep = (32 * (D / 8) % (KB * 2) == 0) ? 32 : BwdStep<KB>::value;
+  static constexpr int kKeyGroups = KB / 32;       // 32 keys per wave
+  static constexpr int kRoleThreads = KB * 2;      // one wave per key group in each of the two roles
+  static constexpr int kThreads = KB * 4;
+  static constexpr int kStep = 32;                 // query rows per step
   static constexpr int kTileElems = kStep * D;
-  static constexpr int kMaxBitmapWords = 4096;      // 64-slot words of the match bitmap (32 KiB)
-  // four tiles (Q and dO, each row-wise and transposed) or the output staging, + lse and delta of a
-  // step's rows, + the bitmap of (query block, slot) pairs that list this KV block
-  static constexpr size_t kTileBytes = (4 * kTileElems > KB * D ? 4 * kTileElems : KB * D) * sizeof(uint16_t);
-  static constexpr size_t kLdsBytes = kTileBytes + 2 * kStep * sizeof(float) + size_t(kMaxBitmapWords) * 8;
+  static constexpr int kMaxBitmapWords = 4096;     // 64-slot words of the match bitmap
+  // two sets of four tiles (Q and dO, each row-wise and transposed; the output staging overlaps
+  // them); two sets of the weights one role hands to the other (fp32, [key group][16][64 lanes]);
+  // -delta and the exponent offsets of the rows of two steps; per 64-slot word of a slab's
+  // metadata the bitmap of the slots that list this KV block and mode / tile index of the first
+  static constexpr size_t kTileBytes = size_t(8) * kTileElems * sizeof(uint16_t);
+  static constexpr size_t kWeightBytes = size_t(2) * kKeyGroups * 16 * 64 * sizeof(float);
+  static constexpr size_t kLdsBytes =
+      kTileBytes + kWeightBytes + 4 * kStep * sizeof(float) + size_t(kMaxBitmapWords) * (8 + 4);
 };
 
-template <bool BF16, int D, int QB, int KB>
-__global__ void __launch_bounds__(KB * 2, 1) bwd_dkdv_kernel(const BwdParams p) {
+// One workgroup per KV block, two waves per 32 keys with different work, so that two waves
+// share each SIMD and the vector work of one runs under the matrix work of the other:
+//   the "weight" wave of a key group holds K, computes S = Q.K^T and P for a step, hands P
+//   (times the soft-cap derivative factor, when capped) to its partner through LDS, and
+//   accumulates dV^T += dO^T.P;
+//   the "gradient" wave holds V, computes dP - delta = dO.V^T - delta, and one step later
+//   dS = P (dP - delta) and dK^T += Q^T.dS.
+// The gradient waves run one step behind the weight waves, so one barrier per step orders
+// the hand-over, the tile loads (each role loads the two tiles it reads) and the reuse of the
+// two buffer sets.
+template <bool BF16, bool CAP, int D, int QB, int KB>
+__global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) {
   using Traits = BwdDkdvTraits<D, KB>;
-  constexpr int NT = Traits::kThreads;
-  constexpr int NW = NT / 64;
+  constexpr int NKG = Traits::kKeyGroups;
+  constexpr int RT = Traits::kRoleThreads;
+  constexpr int NW = Traits::kThreads / 64;
   constexpr int STEP = Traits::kStep;
-  constexpr int SPQ = QB / STEP;  // steps per query block (QB 64 with 64-row steps: one step, half used)
-  constexpr int NSTEPS = SPQ > 0 ? SPQ : 1;
-  constexpr int NTL = STEP / 32;
+  constexpr int NSTEPS = QB / STEP;  // steps per query block
+  constexpr int NTL = 1;
   constexpr int KS = D / 16;
   constexpr int DT = D / 32;
   constexpr int TILE = Traits::kTileElems;
+  constexpr int NTR = (STEP / 16) * DT;  // fragments of the second product
 
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-  uint16_t* sQa = reinterpret_cast<uint16_t*>(lds_raw);
-  uint16_t* sQt = sQa + TILE;
-  uint16_t* sDa = sQt + TILE;
-  uint16_t* sDt = sDa + TILE;
-  float* sLse = reinterpret_cast<float*>(lds_raw + Traits::kTileBytes);
-  float* sDelta = sLse + STEP;
-  uint64_t* sMatch = reinterpret_cast<uint64_t*>(sDelta + STEP);
+  uint16_t* const lds16 = reinterpret_cast<uint16_t*>(lds_raw);  // [2 sets][Qa, Qt, Da, Dt][TILE]
+  float* const sW = reinterpret_cast<float*>(lds_raw + Traits::kTileBytes);  // [2 sets][NKG][16][64]
+  float* const sNd = sW + 2 * NKG * 16 * 64;                                 // [2 sets][STEP] -delta
+  float* const sL2 = sNd + 2 * STEP;                                         // [2 sets][STEP] exponent offsets
+  uint64_t* const sMatch = reinterpret_cast<uint64_t*>(sL2 + 2 * STEP);
+  int32_t* const sFirst = reinterpret_cast<int32_t*>(sMatch + Traits::kMaxBitmapWords);
 
   const int bh = blockIdx.x / p.Tk;
   const int kvb = blockIdx.x - bh * p.Tk;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool grad_role = w >= NKG;        // wave-uniform
+  const int kg = grad_role ? w - NKG : w;  // key group of the wave
+  const int rtid = tid - (grad_role ? RT : 0);
   const int g = lane >> 5, c = lane & 31;
 
   const size_t slab = size_t(bh) * size_t(p.S) * D;
   const uint32_t slab_bytes = uint32_t(p.S) * uint32_t(D * 2);
   const i32x4_t rQ = make_buffer_resource(p.q + slab, slab_bytes);
   const i32x4_t rD = make_buffer_resource(p.dout + slab, slab_bytes);
-  const int key_wave_min = kvb * KB + 32 * w;
+  const i32x4_t rNd = make_buffer_resource(p.ws + size_t(bh) * p.S, uint32_t(p.S) * 4u);
+  const i32x4_t rL2 = make_buffer_resource(p.ws + size_t(p.n_slabs) * p.S + size_t(bh) * p.S, uint32_t(p.S) * 4u);
+  const int key_wave_min = kvb * KB + 32 * kg;
   const int key = key_wave_min + c;  // this lane's key row inside the slab
   const int kr = key < p.S ? key : p.S - 1;
   const bool has_partial = p.partial_idx != nullptr && (p.partial_masks != nullptr || p.partial_bits != nullptr);
   const size_t meta_slab = size_t(bh) * p.Tq;
   const int chunks = (p.max_blocks + 63) / 64;  // 64-slot words per query block
+  const int n_words = p.Tq * chunks;
 
-  // K and V of this lane's key as B operands.
-  u32x4_t kf[KS], vf[KS];
+  // This lane's key as B operand: K for a weight wave, V for a gradient wave.
+  u32x4_t bop[KS];
   {
-    const uint16_t* kp = p.k + slab + size_t(kr) * D + 8 * g;
-    const uint16_t* vp = p.v + slab + size_t(kr) * D + 8 * g;
+    const uint16_t* src = (grad_role ? p.v : p.k) + slab + size_t(kr) * D + 8 * g;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      kf[s] = *reinterpret_cast<const u32x4_t*>(kp + 16 * s);
-      vf[s] = *reinterpret_cast<const u32x4_t*>(vp + 16 * s);
-    }
+    for (int s = 0; s < KS; ++s) bop[s] = *reinterpret_cast<const u32x4_t*>(src + 16 * s);
   }
 
   // Pass 1: which (query block, slot) pairs list this KV block (after the forward's clamping of
   // the block index) with a type the forward would visit?  One 64-bit word per query block and 64
-  // slots; a wave takes one word at a time.
-  for (int word = w; word < p.Tq * chunks; word += NW) {
+  // slots; a wave takes one word at a time.  Mode and tile index of a word's first match are
+  // kept beside it (a list names a block once, except for duplicates and clamped indices).
+  for (int word = w; word < n_words; word += NW) {
     const int qb = word / chunks, ch = word - qb * chunks;
     int nb = load_uniform(p.kv_num_blocks + meta_slab + qb);
     nb = nb < 0 ? 0 : (nb > p.max_blocks ? p.max_blocks : nb);
     const int slot = ch * 64 + lane;
     bool hit = false;
+    int32_t info = 0;
     if (slot < nb) {
       const size_t o = (meta_slab + qb) * p.max_blocks + slot;
       const int32_t raw = p.kv_indices[o];
       const int32_t idx = raw < 0 ? 0 : (raw >= p.Tk ? p.Tk - 1 : raw);
       const int32_t ty = p.types[o];
       const int32_t pid = has_partial ? p.partial_idx[o] : -1;
-      hit = idx == kvb && bwd_slot_mode(ty, pid, has_partial, p.num_partial) != kMasked;
+      const int32_t mode = bwd_slot_mode(ty, pid, has_partial, p.num_partial);
+      hit = idx == kvb && mode != kMasked;
+      info = (mode == kPartial ? pid << 2 : 0) | mode;
     }
     const uint64_t bits = __builtin_amdgcn_ballot_w64(hit);
     if (lane == 0) sMatch[word] = bits;
+    if (bits != 0 && lane == __builtin_ctzll(bits)) sFirst[word] = info;
   }
   __syncthreads();
 
   const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  f32x16_t dk[DT], dv[DT];
+  f32x16_t acc[DT];  // dV^T of a weight wave, dK^T of a gradient wave
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) {
-    dk[dt] = zero16;
-    dv[dt] = zero16;
-  }
+  for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16;
   const bool key_live = key < p.seqlen;
 
-  // Pass 2: visit the matches in ascending (query block, slot) order.
-  for (int word = 0; word < p.Tq * chunks; ++word) {
-    uint64_t bits = sMatch[word];
-    // (readfirstlane returns a signed int: go through uint32_t so that bit 31 does not sign-extend)
-    bits = (uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(bits >> 32))))) << 32) |
-           uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(bits)))));
-    const int qb = word / chunks, ch = word - qb * chunks;
-    while (bits != 0) {
-      const int b = __builtin_ctzll(bits);
-      bits &= bits - 1;
-      const size_t o = (meta_slab + qb) * p.max_blocks + ch * 64 + b;
-      const int32_t ty = load_uniform(p.types + o);
-      const int32_t pid = has_partial ? load_uniform(p.partial_idx + o) : -1;
-      const int32_t mode = bwd_slot_mode(ty, pid, has_partial, p.num_partial);
-      for (int half = 0; half < NSTEPS; ++half) {
-        const int q0 = qb * QB + half * STEP;  // first query row of the step
-        if (q0 >= p.seqlen) continue;
-        if (mode == kCausal && q0 + STEP - 1 < kvb * KB) continue;  // entirely above the diagonal
-        __syncthreads();
-        bwd_load_tile<D, NT, STEP, false>(rQ, q0, lds_offset_of(sQa), tid, w);
-        bwd_load_tile<D, NT, STEP, true>(rQ, q0, lds_offset_of(sQt), tid, w);
-        bwd_load_tile<D, NT, STEP, false>(rD, q0, lds_offset_of(sDa), tid, w);
-        bwd_load_tile<D, NT, STEP, true>(rD, q0, lds_offset_of(sDt), tid, w);
-        if (tid < STEP) {
-          const int row = q0 + tid;
-          // rows of another query block (a 64-row block in a 64-row step never has any), rows
-          // beyond the sequence and rows without any allowed key take no part
-          const bool in_block = row < qb * QB + QB && row < p.seqlen;
-          const float l = in_block ? p.lse[size_t(bh) * p.S + row] : -INFINITY;
-          sLse[tid] = l == -INFINITY ? INFINITY : l * 1.4426950408889634f;
-          sDelta[tid] = in_block ? p.delta[size_t(bh) * p.S + row] : 0.f;
+  // Pass 2: the matches in ascending (query block, slot) order, each as NSTEPS steps of STEP
+  // query rows, skipping steps beyond the sequence and CAUSAL steps entirely above the diagonal.
+  int gw = -1, gsub = 0, g_mode = kMasked, g_pid = -1;
+  uint64_t gbits = 0;
+  bool g_first = true;
+  auto next_step = [&]() {
+    BwdStepInfo st = {0, kMasked, -1, 0, 0, false};
+    for (;;) {
+      if (gsub == 0) {
+        while (gbits == 0) {
+          if (++gw >= n_words) return st;
+          const uint64_t m = sMatch[gw];
+          // (readfirstlane returns a signed int: go through uint32_t so that bit 31 does not sign-extend)
+          gbits = (uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(m >> 32))))) << 32) |
+                  uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(m)))));
+          g_first = true;
         }
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        __syncthreads();
-
-        // S = Q.K^T and dP = dO.V^T : lane = key, registers = query rows
-        f32x16_t sc[NTL], dp[NTL];
-        static_for<NTL>([&](auto tc) {
-          constexpr int t = decltype(tc)::value;
-          sc[t] = zero16;
-          dp[t] = zero16;
-          static_for<KS>([&](auto ks) {
-            constexpr int s = decltype(ks)::value;
-            sc[t] = mfma_32x32x16<BF16>(bwd_row_frag<D>(sQa, s, t, g, c), kf[s], sc[t]);
-            dp[t] = mfma_32x32x16<BF16>(bwd_row_frag<D>(sDa, s, t, g, c), vf[s], dp[t]);
-          });
-        });
-        u32x4_t pb[NTL][2], dsb[NTL][2];
-        static_for<NTL * 4>([&](auto ic) {
-          constexpr int t = decltype(ic)::value / 4, i4 = decltype(ic)::value % 4;
-          // registers 4 i4 .. +3 of tile t are query rows 32 t + 8 i4 + 4 g .. +3 of the step
-          const int ql = 32 * t + 8 * i4 + 4 * g;
-          const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(sLse + ql);
-          const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(sDelta + ql);
-          float pv[4], dsv[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int qrow = q0 + ql + e;  // global query row
-            bool keep = key_live;
-            if (mode == kCausal) keep = keep && key <= qrow;
-            if (mode == kPartial) {
-              const int q_local = qrow - qb * QB, k_local = key - kvb * KB;
-              bool bit = false;
-              if (q_local < QB && key < p.S) {
-                if (p.partial_bits != nullptr) {
-                  bit = (p.partial_bits[(size_t(pid) * QB + q_local) * (KB / 32) + k_local / 32] >> (k_local & 31)) & 1u;
-                } else {
-                  bit = p.partial_masks[(size_t(pid) * QB + q_local) * KB + k_local] != 0;
-                }
-              }
-              keep = keep && bit;
-            }
-            float wgt, fac;
-            bwd_weight(sc[t][4 * i4 + e], l4[e], p, wgt, fac);
-            pv[e] = keep ? wgt : 0.f;
-            dsv[e] = pv[e] * (dp[t][4 * i4 + e] - d4[e]) * fac;
-          }
-          pb[t][i4 >> 1][2 * (i4 & 1) + 0] = pack2<BF16>(pv[0], pv[1]);
-          pb[t][i4 >> 1][2 * (i4 & 1) + 1] = pack2<BF16>(pv[2], pv[3]);
-          dsb[t][i4 >> 1][2 * (i4 & 1) + 0] = pack2<BF16>(dsv[0], dsv[1]);
-          dsb[t][i4 >> 1][2 * (i4 & 1) + 1] = pack2<BF16>(dsv[2], dsv[3]);
-        });
-        // dV^T += dO^T.P and dK^T += Q^T.dS
-        static_for<(STEP / 16) * DT>([&](auto jc) {
-          constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
-          dv[dt] = mfma_32x32x16<BF16>(bwd_tr_frag<D>(sDt, ts, dt, g, c), pb[ts >> 1][ts & 1], dv[dt]);
-          dk[dt] = mfma_32x32x16<BF16>(bwd_tr_frag<D>(sQt, ts, dt, g, c), dsb[ts >> 1][ts & 1], dk[dt]);
-        });
+        const int qb = gw / chunks, ch = gw - qb * chunks;
+        if (g_first) {
+          const int32_t info = __builtin_amdgcn_readfirstlane(sFirst[gw]);
+          g_mode = info & 3;
+          g_pid = g_mode == kPartial ? info >> 2 : -1;
+        } else {  // a further match in the same 64 slots
+          const size_t o = (meta_slab + qb) * p.max_blocks + ch * 64 + __builtin_ctzll(gbits);
+          const int32_t ty = load_uniform(p.types + o);
+          g_pid = has_partial ? load_uniform(p.partial_idx + o) : -1;
+          g_mode = bwd_slot_mode(ty, g_pid, has_partial, p.num_partial);
+        }
       }
+      const int qb = gw / chunks;
+      const int sub = gsub;
+      if (++gsub == NSTEPS) {
+        gsub = 0;
+        gbits &= gbits - 1;
+        g_first = false;
+      }
+      const int q0 = qb * QB + sub * STEP;
+      if (q0 >= p.seqlen) continue;
+      if (g_mode == kCausal && q0 + STEP - 1 < kvb * KB) continue;
+      st.row0 = q0;
+      st.mode = g_mode;
+      st.pid = g_pid;
+      st.blk = qb;
+      st.sub = sub;
+      st.valid = true;
+      return st;
     }
+  };
+  const uint32_t lds_tiles = lds_offset_of(lds16);
+  const uint32_t lds_w = lds_offset_of(sW) + uint32_t(kg) * 4096u + uint32_t(lane) * 16u;
+  const uint32_t lds_nd = lds_offset_of(sNd), lds_l2 = lds_offset_of(sL2);
+  auto tile_at = [&](int set, int which) { return lds_tiles + uint32_t(set * 4 + which) * (TILE * 2u); };
+  // Each role loads what it reads: row-wise Q, transposed dO and the exponent offsets (weight
+  // waves); row-wise dO, transposed Q and -delta (gradient waves).
+  auto load_weight_tiles = [&](const BwdStepInfo& st, int set) {
+    bwd_load_tile<D, RT, STEP, false>(rQ, st.row0, tile_at(set, 0), rtid, kg);
+    bwd_load_tile<D, RT, STEP, true>(rD, st.row0, tile_at(set, 3), rtid, kg);
+    if (rtid < STEP)
+      buffer_to_lds_b32(rL2, uint32_t(rtid) * 4u, uint32_t(st.row0) * 4u, lds_l2 + uint32_t(set * STEP) * 4u);
+  };
+  auto load_grad_tiles = [&](const BwdStepInfo& st, int set) {
+    bwd_load_tile<D, RT, STEP, false>(rD, st.row0, tile_at(set, 2), rtid, kg);
+    bwd_load_tile<D, RT, STEP, true>(rQ, st.row0, tile_at(set, 1), rtid, kg);
+    if (rtid < STEP)
+      buffer_to_lds_b32(rNd, uint32_t(rtid) * 4u, uint32_t(st.row0) * 4u, lds_nd + uint32_t(set * STEP) * 4u);
+  };
+  const uint32_t row_lane = bwd_row_lane<D>(g, c);
+  const uint32_t tr_lane = bwd_tr_lane<D>(g, c);
+
+  // Weight wave, one step: S = Q.K^T (lane = key, registers = query rows), P, dV^T += dO^T.P.
+  auto weight_step = [&](int set, uint32_t kw) {
+    const uint32_t aQ = tile_at(set, 0) + row_lane, tD = tile_at(set, 3) + tr_lane;
+    u32x4_t fa[KS];
+    static_for<KS>([&](auto ks) {
+      constexpr int s = decltype(ks)::value;
+      fa[s] = lds_b128_at(aQ ^ uint32_t(32 * s));
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    f32x16_t sc = zero16;
+    static_for<KS>([&](auto ks) {
+      constexpr int s = decltype(ks)::value;
+      sc = mfma_32x32x16<BF16>(fa[s], bop[s], sc);
+    });
+    u32x4_t gd[NTR];
+    static_for<NTR>([&](auto jc) {
+      constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
+      gd[ts * DT + dt] = lds_tr_pair_at((tD ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u, 8u * D * 2u);
+    });
+    f32x4_t l4[4];
+    static_for<4>([&](auto ic) {
+      constexpr int i4 = decltype(ic)::value;
+      // registers 4 i4 .. +3 are query rows 8 i4 + 4 g .. +3 of the step
+      l4[i4] = lds_f32x4_at(lds_l2 + uint32_t(set * STEP + 8 * i4) * 4u + 16u * g);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    u32x4_t pb[2];
+    static_for<4>([&](auto ic) {
+      constexpr int i4 = decltype(ic)::value;
+      float pv[4];
+      f32x4_t hand;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool keep = (kw >> (8 * i4 + e)) & 1u;  // (kw is already shifted by 4 g)
+        float wgt, fac;
+        bwd_weight<CAP>(sc[4 * i4 + e], l4[i4][e], p, wgt, fac);
+        pv[e] = keep ? wgt : 0.f;
+        hand[e] = pv[e] * fac;
+      }
+      *(__attribute__((address_space(3))) f32x4_t*)(lds_w + uint32_t(set) * (NKG * 4096u) + uint32_t(i4) * 1024u) = hand;
+      pb[i4 >> 1][2 * (i4 & 1) + 0] = pack2<BF16>(pv[0], pv[1]);
+      pb[i4 >> 1][2 * (i4 & 1) + 1] = pack2<BF16>(pv[2], pv[3]);
+    });
+    static_for<NTR>([&](auto jc) {
+      constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
+      acc[dt] = mfma_32x32x16<BF16>(gd[ts * DT + dt], pb[ts], acc[dt]);
+    });
+  };
+  // Gradient wave, one step: dP - delta = dO.V^T - delta (the accumulator starts at -delta),
+  // dS = P (dP - delta) with the partner's P, dK^T += Q^T.dS.
+  auto grad_step = [&](int set) {
+    const uint32_t aD = tile_at(set, 2) + row_lane, tQ = tile_at(set, 1) + tr_lane;
+    f32x16_t dp;
+    static_for<4>([&](auto ic) {
+      constexpr int i4 = decltype(ic)::value;
+      const f32x4_t nd = lds_f32x4_at(lds_nd + uint32_t(set * STEP + 8 * i4) * 4u + 16u * g);
+      dp[4 * i4 + 0] = nd[0];
+      dp[4 * i4 + 1] = nd[1];
+      dp[4 * i4 + 2] = nd[2];
+      dp[4 * i4 + 3] = nd[3];
+    });
+    u32x4_t fb[KS];
+    static_for<KS>([&](auto ks) {
+      constexpr int s = decltype(ks)::value;
+      fb[s] = lds_b128_at(aD ^ uint32_t(32 * s));
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<KS>([&](auto ks) {
+      constexpr int s = decltype(ks)::value;
+      dp = mfma_32x32x16<BF16>(fb[s], bop[s], dp);
+    });
+    u32x4_t gq[NTR];
+    static_for<NTR>([&](auto jc) {
+      constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
+      gq[ts * DT + dt] = lds_tr_pair_at((tQ ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u, 8u * D * 2u);
+    });
+    f32x4_t hand[4];
+    static_for<4>([&](auto ic) {
+      constexpr int i4 = decltype(ic)::value;
+      hand[i4] = lds_f32x4_at(lds_w + uint32_t(set) * (NKG * 4096u) + uint32_t(i4) * 1024u);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    u32x4_t dsb[2];
+    static_for<4>([&](auto ic) {
+      constexpr int i4 = decltype(ic)::value;
+      dsb[i4 >> 1][2 * (i4 & 1) + 0] = pack2<BF16>(hand[i4][0] * dp[4 * i4 + 0], hand[i4][1] * dp[4 * i4 + 1]);
+      dsb[i4 >> 1][2 * (i4 & 1) + 1] = pack2<BF16>(hand[i4][2] * dp[4 * i4 + 2], hand[i4][3] * dp[4 * i4 + 3]);
+    });
+    static_for<NTR>([&](auto jc) {
+      constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
+      acc[dt] = mfma_32x32x16<BF16>(gq[ts * DT + dt], dsb[ts], acc[dt]);
+    });
+  };
+
+  // Bits of one partial tile for this lane's key: bit j = query row q_local0 + j of the tile
+  // attends the key.  Lane j of the wave fetches the 32 key bits of row j; the column of this
+  // lane's key is then collected from the 32 rows.
+  auto partial_column = [&](int pid, int q_local0) {
+    const int rl = lane & 31;
+    uint32_t roww;
+    if (p.partial_bits != nullptr) {
+      roww = p.partial_bits[(size_t(pid) * QB + q_local0 + rl) * (KB / 32) + kg];
+    } else {
+      const uint8_t* mp = p.partial_masks + (size_t(pid) * QB + q_local0 + rl) * KB + 32 * kg;
+      roww = bwd_pack32(*reinterpret_cast<const u32x4_t*>(mp), *reinterpret_cast<const u32x4_t*>(mp + 16));
+    }
+    uint32_t col = 0;
+    static_for<32>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      const uint32_t r = uint32_t(__builtin_amdgcn_readlane(int(roww), j));
+      col |= ((r >> c) & 1u) << j;
+    });
+    return col;
+  };
+
+  // Iteration j: the weight waves do step j, the gradient waves step j - 1.  The two roles
+  // run separate copies of the loop (same trip count, one barrier per trip), so that each keeps
+  // its accumulators in place.
+  auto run = [&](auto role_c) {
+    constexpr bool GRAD = decltype(role_c)::value;
+    const BwdStepInfo none = {0, kMasked, -1, 0, 0, false};
+    BwdStepInfo prev = none, cur = next_step();
+    if constexpr (!GRAD) {
+      if (cur.valid) load_weight_tiles(cur, 0);
+    }
+    for (int j = 0; cur.valid || prev.valid; ++j) {
+      const BwdStepInfo nxt = cur.valid ? next_step() : none;
+      // mask word of this lane's key: bit i = query row row0 + i attends it
+      uint32_t kw = 0;
+      if constexpr (!GRAD) {
+        if (cur.valid) {
+          uint32_t m = key_live ? 0xffffffffu : 0u;
+          if (cur.mode == kCausal) {  // rows at or after the key
+            const int n = key - cur.row0;
+            m &= n <= 0 ? 0xffffffffu : (n >= 32 ? 0u : (0xffffffffu << (n & 31)));
+          }
+          if (cur.mode == kPartial) m &= partial_column(cur.pid, cur.row0 - cur.blk * QB);
+          kw = m >> (4 * g);
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the tiles this wave loaded have landed
+      __syncthreads();  // ... everybody's have; the hand-over of step j - 1 is written; the sets
+                        // about to be overwritten are no longer read
+      if constexpr (!GRAD) {
+        if (nxt.valid) load_weight_tiles(nxt, (j + 1) & 1);
+        if (cur.valid) weight_step(j & 1, kw);
+      } else {
+        if (cur.valid) load_grad_tiles(cur, j & 1);
+        if (prev.valid) grad_step((j + 1) & 1);
+      }
+      prev = cur;
+      cur = nxt;
+    }
+    __syncthreads();
+    uint16_t* stage = lds16 + size_t(w) * 32 * D;
+    if constexpr (!GRAD) {
+      bwd_store_rows<BF16, D>(acc, 1.f, stage, p.dv + slab, key_wave_min, p.S, lane);
+    } else {
+      bwd_store_rows<BF16, D>(acc, p.scale, stage, p.dk + slab, key_wave_min, p.S, lane);
+    }
+  };
+  if (grad_role) {
+    run(std::integral_constant<bool, true>{});
+  } else {
+    run(std::integral_constant<bool, false>{});
   }
-  __syncthreads();
-  uint16_t* stage = reinterpret_cast<uint16_t*>(lds_raw) + size_t(w) * 32 * D;
-  bwd_store_rows<BF16, D>(dk, p.scale, stage, p.dk + slab, key_wave_min, p.S, lane);
-  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the staging reads of dK are done before dV overwrites them
-  bwd_store_rows<BF16, D>(dv, 1.f, stage, p.dv + slab, key_wave_min, p.S, lane);
 }
 
 constexpr int kBwdMaxDevices = 64;
 
-template <bool BF16, int D, int QB, int KB>
-int launch_bwd(const BwdParams& p, hipStream_t stream) {
+template <bool BF16, bool CAP, int D, int QB, int KB>
+int launch_bwd_cap(const BwdParams& p, hipStream_t stream) {
   using TQ = BwdDqTraits<D, QB>;
   using TK = BwdDkdvTraits<D, KB>;
-  auto kq = bwd_dq_kernel<BF16, D, QB, KB>;
-  auto kk = bwd_dkdv_kernel<BF16, D, QB, KB>;
+  auto kq = bwd_dq_kernel<BF16, CAP, D, QB, KB>;
+  auto kk = bwd_dkdv_kernel<BF16, CAP, D, QB, KB>;
   static std::atomic<bool> lds_limit_set[kBwdMaxDevices];
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -575,6 +867,14 @@ int launch_bwd(const BwdParams& p, hipStream_t stream) {
   e = hipLaunchKernel(reinterpret_cast<const void*>(kk), dim3(unsigned(p.n_slabs) * unsigned(p.Tk)),
                       dim3(TK::kThreads), args, TK::kLdsBytes, stream);
   return int(e);
+}
+
+// The soft-capped instances are separate kernels: the extra arithmetic per score would
+// otherwise cost the plain ones registers.
+template <bool BF16, int D, int QB, int KB>
+int launch_bwd(const BwdParams& p, hipStream_t stream) {
+  return p.softcap > 0.f ? launch_bwd_cap<BF16, true, D, QB, KB>(p, stream)
+                         : launch_bwd_cap<BF16, false, D, QB, KB>(p, stream);
 }
 
 }  // namespace omni_attn

@@ -197,7 +197,8 @@ extern "C" int omni_attn_fwd_packed_gfx950(const void* q, const void* k, const v
 
 extern "C" size_t omni_attn_bwd_workspace_bytes(int B, int H, int S_pad) {
   if (B <= 0 || H <= 0 || S_pad <= 0) return 0;
-  return size_t(B) * size_t(H) * size_t(S_pad) * sizeof(float);  // delta = rowsum(dO . O)
+  // two floats per row: -rowsum(dO . O) and the row's exponent offset
+  return size_t(B) * size_t(H) * size_t(S_pad) * 2 * sizeof(float);
 }
 
 namespace {
@@ -246,7 +247,7 @@ int backward(const void* q, const void* k, const void* v, const void* o, const v
   p.dq = static_cast<uint16_t*>(dq);
   p.dk = static_cast<uint16_t*>(dk);
   p.dv = static_cast<uint16_t*>(dv);
-  p.delta = delta_workspace;
+  p.ws = delta_workspace;
   p.kv_num_blocks = kv_num_blocks;
   p.kv_indices = kv_indices;
   p.types = block_mask_types;
@@ -301,9 +302,10 @@ extern "C" int omni_attn_bwd_gfx950(const void* q, const void* k, const void* v,
 }
 
 // ---- the backward for callers that cannot allocate -------------------------------------------
-// Same kernels; the delta workspace is this file-scope device array instead of caller memory.
+// Same kernels; the workspace (two floats per row) is this file-scope device array instead of
+// caller memory.
 // Every GPU the library runs on holds its own copy at its own address until the process ends.
-constexpr size_t kScratchFloats = size_t(4) << 20;  // 16 MiB: B * H * S_pad up to 4 194 304 rows
+constexpr size_t kScratchFloats = size_t(8) << 20;  // 32 MiB: B * H * S_pad up to 4 194 304 rows
 static __device__ __align__(256) float scratch[kScratchFloats];
 
 namespace {
@@ -330,7 +332,7 @@ int scratch_address(float** out) {
 }
 }  // namespace
 
-extern "C" size_t omni_attn_bwd_noalloc_max_rows(void) { return kScratchFloats; }
+extern "C" size_t omni_attn_bwd_noalloc_max_rows(void) { return kScratchFloats / 2; }
 
 extern "C" int omni_attn_bwd_noalloc_gfx950(const void* q, const void* k, const void* v, const void* o,
                                             const void* dout, const float* lse, void* dq, void* dk,
@@ -342,15 +344,15 @@ extern "C" int omni_attn_bwd_noalloc_gfx950(const void* q, const void* k, const 
                                             int D, int Tq, int max_blocks, int QB, int KB, int num_partial,
                                             int seqlen_orig, int dtype, float softcap, void* stream) {
   if (B <= 0 || H <= 0 || S_pad <= 0) return OMNI_ATTN_ERR_BAD_SHAPE;
-  if ((unsigned long long)B * (unsigned long long)H * (unsigned long long)S_pad > kScratchFloats)
+  if ((unsigned long long)B * (unsigned long long)H * (unsigned long long)S_pad > kScratchFloats / 2)
     return OMNI_ATTN_ERR_SCRATCH_LIMIT;
   float* delta = nullptr;
   if (const int e = scratch_address(&delta)) {
     g_last_hip_error = e;
     return OMNI_ATTN_ERR_LAUNCH;
   }
-  // Nothing in the array has to start at zero: the dQ kernel writes delta for every row of every
-  // slab before the dK/dV kernel, which runs after it on the same stream, reads any of them.
+  // Nothing in the array has to start at zero: the dQ kernel writes both floats of every row of
+  // every slab before the dK/dV kernel, which runs after it on the same stream, reads any of them.
   return backward(q, k, v, o, dout, lse, dq, dk, dv, kv_num_blocks, kv_indices, block_mask_types,
                   partial_idx_or_null, partial_masks_or_null, partial_bits_or_null, delta, B, H, S_pad, D,
                   Tq, max_blocks, QB, KB, num_partial, seqlen_orig, dtype, softcap, stream);

@@ -140,7 +140,7 @@ def test_backward_is_bitwise_reproducible_and_checks_its_workspace(gpu_device):
     for x, y in zip(a[:3], b[:3]):
         assert torch.equal(x, y)
     lib = omni_attn_capi.load_library()
-    assert lib.omni_attn_bwd_workspace_bytes(1, 2, 1024) == 1 * 2 * 1024 * 4
+    assert lib.omni_attn_bwd_workspace_bytes(1, 2, 1024) == 1 * 2 * 1024 * 2 * 4
     small = torch.empty(16, dtype=torch.uint8, device=gpu_device)
     q = w.q.to(gpu_device)
     with pytest.raises(RuntimeError, match="workspace"):
