@@ -55,6 +55,7 @@ struct BwdParams {
   const uint32_t* partial_bits;
   int num_partial;
   int S, Tq, Tk, max_blocks, seqlen, n_slabs;
+  int n_xcd;      // XCDs (L2 domains) of the device; workgroup ids go round-robin over them
   float sl2;      // log2(e) / sqrt(D)
   float scale;    // 1 / sqrt(D)
   float softcap;  // > 0: the forward replaced x = s / sqrt(D) by softcap * tanh(x / softcap)
@@ -252,8 +253,14 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
   uint16_t* const lds16 = reinterpret_cast<uint16_t*>(lds_raw);  // [2 sets][Ka, Kt, Va][TILE]
 
-  const int bh = blockIdx.x / p.Tq;
-  const int qb = p.Tq - 1 - (blockIdx.x - bh * p.Tq);
+  // Workgroup -> (slab, query block): XCD x takes the slabs bh with bh % n_xcd == x one after
+  // the other, longest query block first, so the workgroups that run together on an XCD walk the
+  // K/V rows of one or two slabs and share them through that XCD's L2.
+  const int slot = blockIdx.x / p.n_xcd;
+  const int xcd = blockIdx.x - slot * p.n_xcd;
+  if (slot >= ((p.n_slabs - xcd + p.n_xcd - 1) / p.n_xcd) * p.Tq) return;
+  const int bh = xcd + p.n_xcd * (slot / p.Tq);
+  const int qb = p.Tq - 1 - slot % p.Tq;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -535,8 +542,14 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
   uint64_t* const sMatch = reinterpret_cast<uint64_t*>(sL2 + 2 * STEP);
   int32_t* const sFirst = reinterpret_cast<int32_t*>(sMatch + Traits::kMaxBitmapWords);
 
-  const int bh = blockIdx.x / p.Tk;
-  const int kvb = blockIdx.x - bh * p.Tk;
+  // Workgroup -> (slab, KV block): XCD x takes the slabs bh with bh % n_xcd == x one after the
+  // other, so the workgroups that run together on an XCD read the Q and dO rows of one slab and
+  // share them through that XCD's L2.
+  const int slot = blockIdx.x / p.n_xcd;
+  const int xcd = blockIdx.x - slot * p.n_xcd;
+  if (slot >= ((p.n_slabs - xcd + p.n_xcd - 1) / p.n_xcd) * p.Tk) return;
+  const int bh = xcd + p.n_xcd * (slot / p.Tk);
+  const int kvb = slot % p.Tk;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -602,7 +615,7 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
 
   // Pass 2: the matches in ascending (query block, slot) order, each as NSTEPS steps of STEP
   // query rows, skipping steps beyond the sequence and CAUSAL steps entirely above the diagonal.
-  int gw = -1, gsub = 0, g_mode = kMasked, g_pid = -1;
+  int gw = -1, g_qb = 0, g_ch = -1, gsub = 0, g_mode = kMasked, g_pid = -1;  // word gw = (g_qb, g_ch)
   uint64_t gbits = 0;
   bool g_first = true;
   auto next_step = [&]() {
@@ -611,25 +624,28 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
       if (gsub == 0) {
         while (gbits == 0) {
           if (++gw >= n_words) return st;
+          if (++g_ch == chunks) {
+            g_ch = 0;
+            ++g_qb;
+          }
           const uint64_t m = sMatch[gw];
           // (readfirstlane returns a signed int: go through uint32_t so that bit 31 does not sign-extend)
           gbits = (uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(m >> 32))))) << 32) |
                   uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(m)))));
           g_first = true;
         }
-        const int qb = gw / chunks, ch = gw - qb * chunks;
         if (g_first) {
           const int32_t info = __builtin_amdgcn_readfirstlane(sFirst[gw]);
           g_mode = info & 3;
           g_pid = g_mode == kPartial ? info >> 2 : -1;
         } else {  // a further match in the same 64 slots
-          const size_t o = (meta_slab + qb) * p.max_blocks + ch * 64 + __builtin_ctzll(gbits);
+          const size_t o = (meta_slab + g_qb) * p.max_blocks + g_ch * 64 + __builtin_ctzll(gbits);
           const int32_t ty = load_uniform(p.types + o);
           g_pid = has_partial ? load_uniform(p.partial_idx + o) : -1;
           g_mode = bwd_slot_mode(ty, g_pid, has_partial, p.num_partial);
         }
       }
-      const int qb = gw / chunks;
+      const int qb = g_qb;
       const int sub = gsub;
       if (++gsub == NSTEPS) {
         gsub = 0;
@@ -859,12 +875,13 @@ int launch_bwd_cap(const BwdParams& p, hipStream_t stream) {
     if (e != hipSuccess) return int(e);
     if (cached) lds_limit_set[dev].store(true, std::memory_order_release);
   }
+  const unsigned slabs_per_xcd = unsigned(p.n_slabs + p.n_xcd - 1) / unsigned(p.n_xcd);
   BwdParams params = p;
   void* args[] = {&params};
-  e = hipLaunchKernel(reinterpret_cast<const void*>(kq), dim3(unsigned(p.n_slabs) * unsigned(p.Tq)),
+  e = hipLaunchKernel(reinterpret_cast<const void*>(kq), dim3(unsigned(p.n_xcd) * slabs_per_xcd * unsigned(p.Tq)),
                       dim3(TQ::kThreads), args, TQ::kLdsBytes, stream);
   if (e != hipSuccess) return int(e);
-  e = hipLaunchKernel(reinterpret_cast<const void*>(kk), dim3(unsigned(p.n_slabs) * unsigned(p.Tk)),
+  e = hipLaunchKernel(reinterpret_cast<const void*>(kk), dim3(unsigned(p.n_xcd) * slabs_per_xcd * unsigned(p.Tk)),
                       dim3(TK::kThreads), args, TK::kLdsBytes, stream);
   return int(e);
 }

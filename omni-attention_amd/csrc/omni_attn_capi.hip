@@ -263,6 +263,12 @@ int backward(const void* q, const void* k, const void* v, const void* o, const v
   p.max_blocks = max_blocks;
   p.seqlen = seqlen_orig < S_pad ? seqlen_orig : S_pad;
   p.n_slabs = B * H;
+  DeviceTopology topo;
+  if (const int e = query_topology(&topo)) {
+    g_last_hip_error = e;
+    return OMNI_ATTN_ERR_LAUNCH;
+  }
+  p.n_xcd = topo.n_xcd;
   p.scale = float(1.0 / std::sqrt(double(D)));
   p.sl2 = float(1.4426950408889634 / std::sqrt(double(D)));
   p.softcap = softcap;
