@@ -385,7 +385,7 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   // One step: S^T = K.Q^T and dP^T = V.dO^T (lane = query row, registers = keys), then
   // dS^T = P^T (dP^T - delta) packed to 16 bits in the order the next product reads it, then
   // dQ^T += K^T.dS^T.
-  auto compute = [&](int set, const uint32_t (&kw)[NTL]) {
+  auto compute = [&](int set, const uint32_t (&kw)[NTL], bool all_allowed) {
     const uint32_t base = lds_tiles + uint32_t(set) * (3u * TILE * 2u);
     const uint32_t aK = base + row_lane, aV = aK + 2u * TILE * 2u, tK = base + TILE * 2u + tr_lane;
     f32x16_t st[NTL], dp[NTL];
@@ -417,20 +417,29 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
     });
     __builtin_amdgcn_sched_barrier(0);
     u32x4_t dsb[NTL][2];
-    static_for<8 * NTL>([&](auto ic) {
-      constexpr int i = decltype(ic)::value;
-      constexpr int t = i / 8, r = 2 * (i % 8);
-      constexpr int kl0 = 8 * (r >> 2) + (r & 3), kl1 = 8 * ((r + 1) >> 2) + ((r + 1) & 3);
-      const bool keep0 = (kw[t] >> kl0) & 1u, keep1 = (kw[t] >> kl1) & 1u;
-      float w0, w1, f0, f1;
-      bwd_weight<CAP>(st[t][r], lse2, p, w0, f0);
-      bwd_weight<CAP>(st[t][r + 1], lse2, p, w1, f1);
-      const float p0 = keep0 ? w0 : 0.f;
-      const float p1 = keep1 ? w1 : 0.f;
-      const float d0 = p0 * (dp[t][r] - delta) * f0;
-      const float d1 = p1 * (dp[t][r + 1] - delta) * f1;
-      dsb[t][r >> 3][(r & 7) >> 1] = pack2<BF16>(d0, d1);
-    });
+    auto weights = [&](auto masked_c) {
+      constexpr bool MASKED = decltype(masked_c)::value;
+      static_for<8 * NTL>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int t = i / 8, r = 2 * (i % 8);
+        constexpr int kl0 = 8 * (r >> 2) + (r & 3), kl1 = 8 * ((r + 1) >> 2) + ((r + 1) & 3);
+        float p0, p1, f0, f1;
+        bwd_weight<CAP>(st[t][r], lse2, p, p0, f0);
+        bwd_weight<CAP>(st[t][r + 1], lse2, p, p1, f1);
+        if constexpr (MASKED) {
+          p0 = ((kw[t] >> kl0) & 1u) ? p0 : 0.f;
+          p1 = ((kw[t] >> kl1) & 1u) ? p1 : 0.f;
+        }
+        const float d0 = p0 * (dp[t][r] - delta) * f0;
+        const float d1 = p1 * (dp[t][r + 1] - delta) * f1;
+        dsb[t][r >> 3][(r & 7) >> 1] = pack2<BF16>(d0, d1);
+      });
+    };
+    if (all_allowed) {  // (wave-uniform) a FULL step inside the sequence needs no mask
+      weights(std::integral_constant<bool, false>{});
+    } else {
+      weights(std::integral_constant<bool, true>{});
+    }
     static_for<NTS>([&](auto tsc) {
       constexpr int ts = decltype(tsc)::value;
       if constexpr (ts + 1 < NTS) {
@@ -483,7 +492,7 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this step's tiles (and mask words) have landed
     __syncthreads();                     // ... for every wave; and the other set is no longer read
     if (nxt.valid) issue_loads(nxt, set ^ 1);
-    compute(set, kw);
+    compute(set, kw, cur.mode == kFull && cur.row0 + STEP <= p.seqlen);
     set ^= 1;
     cur = nxt;
   }
@@ -506,8 +515,11 @@ struct BwdDkdvTraits {
   // metadata the bitmap of the slots that list this KV block and mode / tile index of the first
   static constexpr size_t kTileBytes = size_t(8) * kTileElems * sizeof(uint16_t);
   static constexpr size_t kWeightBytes = size_t(2) * kKeyGroups * 16 * 64 * sizeof(float);
-  static constexpr size_t kLdsBytes =
-      kTileBytes + kWeightBytes + 4 * kStep * sizeof(float) + size_t(kMaxBitmapWords) * (8 + 4);
+  // (the launch asks for the words its metadata needs, so small problems fit two workgroups)
+  static constexpr size_t lds_bytes(size_t bitmap_words) {
+    return kTileBytes + kWeightBytes + 4 * kStep * sizeof(float) + bitmap_words * (8 + 4);
+  }
+  static constexpr size_t kLdsBytes = lds_bytes(kMaxBitmapWords);
 };
 
 // One workgroup per KV block, two waves per 32 keys with different work, so that two waves
@@ -540,7 +552,7 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
   float* const sNd = sW + 2 * NKG * 16 * 64;                                 // [2 sets][STEP] -delta
   float* const sL2 = sNd + 2 * STEP;                                         // [2 sets][STEP] exponent offsets
   uint64_t* const sMatch = reinterpret_cast<uint64_t*>(sL2 + 2 * STEP);
-  int32_t* const sFirst = reinterpret_cast<int32_t*>(sMatch + Traits::kMaxBitmapWords);
+  int32_t* const sFirst = reinterpret_cast<int32_t*>(sMatch + p.Tq * ((p.max_blocks + 63) / 64));
 
   // Workgroup -> (slab, KV block): XCD x takes the slabs bh with bh % n_xcd == x one after the
   // other, so the workgroups that run together on an XCD read the Q and dO rows of one slab and
@@ -686,7 +698,7 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
   const uint32_t tr_lane = bwd_tr_lane<D>(g, c);
 
   // Weight wave, one step: S = Q.K^T (lane = key, registers = query rows), P, dV^T += dO^T.P.
-  auto weight_step = [&](int set, uint32_t kw) {
+  auto weight_step = [&](int set, uint32_t kw, bool all_allowed) {
     const uint32_t aQ = tile_at(set, 0) + row_lane, tD = tile_at(set, 3) + tr_lane;
     u32x4_t fa[KS];
     static_for<KS>([&](auto ks) {
@@ -712,22 +724,30 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
     });
     __builtin_amdgcn_sched_barrier(0);
     u32x4_t pb[2];
-    static_for<4>([&](auto ic) {
-      constexpr int i4 = decltype(ic)::value;
-      float pv[4];
-      f32x4_t hand;
+    auto weights = [&](auto masked_c) {
+      constexpr bool MASKED = decltype(masked_c)::value;
+      static_for<4>([&](auto ic) {
+        constexpr int i4 = decltype(ic)::value;
+        float pv[4];
+        f32x4_t hand;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const bool keep = (kw >> (8 * i4 + e)) & 1u;  // (kw is already shifted by 4 g)
-        float wgt, fac;
-        bwd_weight<CAP>(sc[4 * i4 + e], l4[i4][e], p, wgt, fac);
-        pv[e] = keep ? wgt : 0.f;
-        hand[e] = pv[e] * fac;
-      }
-      *(__attribute__((address_space(3))) f32x4_t*)(lds_w + uint32_t(set) * (NKG * 4096u) + uint32_t(i4) * 1024u) = hand;
-      pb[i4 >> 1][2 * (i4 & 1) + 0] = pack2<BF16>(pv[0], pv[1]);
-      pb[i4 >> 1][2 * (i4 & 1) + 1] = pack2<BF16>(pv[2], pv[3]);
-    });
+        for (int e = 0; e < 4; ++e) {
+          float wgt, fac;
+          bwd_weight<CAP>(sc[4 * i4 + e], l4[i4][e], p, wgt, fac);
+          if constexpr (MASKED) wgt = ((kw >> (8 * i4 + e)) & 1u) ? wgt : 0.f;  // (kw is already shifted by 4 g)
+          pv[e] = wgt;
+          hand[e] = wgt * fac;
+        }
+        *(__attribute__((address_space(3))) f32x4_t*)(lds_w + uint32_t(set) * (NKG * 4096u) + uint32_t(i4) * 1024u) = hand;
+        pb[i4 >> 1][2 * (i4 & 1) + 0] = pack2<BF16>(pv[0], pv[1]);
+        pb[i4 >> 1][2 * (i4 & 1) + 1] = pack2<BF16>(pv[2], pv[3]);
+      });
+    };
+    if (all_allowed) {  // (wave-uniform) a FULL step whose keys are all inside the sequence needs no mask
+      weights(std::integral_constant<bool, false>{});
+    } else {
+      weights(std::integral_constant<bool, true>{});
+    }
     static_for<NTR>([&](auto jc) {
       constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
       acc[dt] = mfma_32x32x16<BF16>(gd[ts * DT + dt], pb[ts], acc[dt]);
@@ -830,7 +850,7 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
                         // about to be overwritten are no longer read
       if constexpr (!GRAD) {
         if (nxt.valid) load_weight_tiles(nxt, (j + 1) & 1);
-        if (cur.valid) weight_step(j & 1, kw);
+        if (cur.valid) weight_step(j & 1, kw, cur.mode == kFull && key_wave_min + 32 <= p.seqlen);
       } else {
         if (cur.valid) load_grad_tiles(cur, j & 1);
         if (prev.valid) grad_step((j + 1) & 1);
@@ -882,7 +902,8 @@ int launch_bwd_cap(const BwdParams& p, hipStream_t stream) {
                       dim3(TQ::kThreads), args, TQ::kLdsBytes, stream);
   if (e != hipSuccess) return int(e);
   e = hipLaunchKernel(reinterpret_cast<const void*>(kk), dim3(unsigned(p.n_xcd) * slabs_per_xcd * unsigned(p.Tk)),
-                      dim3(TK::kThreads), args, TK::kLdsBytes, stream);
+                      dim3(TK::kThreads), args,
+                      TK::lds_bytes(size_t(p.Tq) * size_t((p.max_blocks + 63) / 64)), stream);
   return int(e);
 }
 
