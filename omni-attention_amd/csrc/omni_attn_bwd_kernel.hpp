@@ -87,39 +87,47 @@ __device__ __forceinline__ u32x4_t lds_b128_at(uint32_t addr) {
 __device__ __forceinline__ f32x4_t lds_f32x4_at(uint32_t addr) {
   return *(const __attribute__((address_space(3))) f32x4_t*)(addr);
 }
-__device__ __forceinline__ u32x4_t lds_tr_pair_at(uint32_t addr, uint32_t hi_off) {
-  const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(addr));
-  const s16x4_t hi =
-      __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(addr + hi_off));
+__device__ __forceinline__ u32x4_t lds_tr_pair_at(uint32_t lo_addr, uint32_t hi_addr) {
+  const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(lo_addr));
+  const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(hi_addr));
   const u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo);
   const u32x2_t hi2 = __builtin_bit_cast(u32x2_t, hi);
   const u32x4_t a = {lo2[0], lo2[1], hi2[0], hi2[1]};
   return a;
 }
+
+// One LDS layout serves both kinds of operand reads of a backward tile ([rows][D] 16-bit, the
+// 16-byte chunk index of a row XORed with a function of the row, period 16 rows):
+//   row-wise (ds_read_b128): 16 lanes read the same chunk of 16 consecutive rows -- the 16 XOR
+//   values of 16 consecutive rows put them on 16 different 16-byte bank groups;
+//   transposed (ds_read_b64_tr_b16): 32 lanes read 4 consecutive chunks of 4 consecutive rows
+//   (starting at a multiple of 4) -- those 16 chunks land on 16 different bank groups too.
+// So a tile is loaded once however it is read.
+template <int D>
+__device__ __forceinline__ int bwd_swizzle(int row) {
+  if constexpr (D == 128) return ((row & 3) << 2) | ((row >> 2) & 3);
+  if constexpr (D == 64) return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+  return (row >> 2) & 3;
+}
 // Lane part (bytes) of a row-wise A fragment: row 32 t + c of the tile, k-step s at
 // ((tile + lane part) ^ 32 s) + 32 t rows.
 template <int D>
 __device__ __forceinline__ uint32_t bwd_row_lane(int g, int c) {
-  return uint32_t(c * D + (g ^ k_swizzle<D>(c)) * 8) * 2u;
+  return uint32_t(c * D + (g ^ bwd_swizzle<D>(c)) * 8) * 2u;
 }
 // Lane part (bytes) of a transposed A fragment: rows 32 dt .. +31 of tile^T at tile rows
 // 16 ts .. +15 (taken in the accumulator order of the first product) at
-// ((tile + lane part) ^ 64 dt) + 16 ts rows, second half 8 rows further.
+// ((tile + lane part) ^ 64 dt) + 16 ts rows; `upper` selects the second half, 8 rows further.
 template <int D>
-__device__ __forceinline__ uint32_t bwd_tr_lane(int g, int c) {
-  const int i16 = c & 15, j16 = c >> 4, r0 = 4 * g + (i16 >> 2);
-  return uint32_t(r0 * D + (j16 ^ v_swizzle<D>(r0)) * 16 + (i16 & 3) * 4) * 2u;
+__device__ __forceinline__ uint32_t bwd_tr_lane(int g, int c, int upper) {
+  const int i16 = c & 15, j16 = c >> 4, r = 4 * g + (i16 >> 2) + 8 * upper;
+  const int chunk = 2 * j16 + ((i16 & 3) >> 1);
+  return uint32_t(r * D * 2 + (chunk ^ bwd_swizzle<D>(r)) * 16 + (i16 & 1) * 8);
 }
 
-template <int QB>
-struct BwdStep {
-  // rows of a tile: the forward's rule (a 64-row block has half the threads)
-  static constexpr int value = QB == 64 ? 32 : 64;
-};
-
-// [ROWS][D] tile from a slab into LDS, 16-byte chunks swizzled for row-wise (TR = false) or
-// transposed (TR = true) operand reads.  Rows at or beyond the end of the slab read as zeros.
-template <int D, int NT, int ROWS, bool TR>
+// [ROWS][D] tile from a slab into LDS in that layout.  Rows at or beyond the end of the slab
+// read as zeros.
+template <int D, int NT, int ROWS>
 __device__ __forceinline__ void bwd_load_tile(i32x4_t rsrc, int row0, uint32_t lds_tile, int tid, int w) {
   constexpr int CPR = D / 8;
   constexpr int TOTAL = ROWS * CPR;  // 16-byte chunks of the tile
@@ -131,38 +139,9 @@ __device__ __forceinline__ void bwd_load_tile(i32x4_t rsrc, int row0, uint32_t l
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int row = ld_row + i * ROW_STRIDE;
-    uint32_t off;
-    if constexpr (TR) {
-      off = uint32_t(row * D + ((((ld_pch >> 1) ^ v_swizzle<D>(row)) << 1) | (ld_pch & 1)) * 8) * 2u;
-    } else {
-      off = uint32_t(row * D + (ld_pch ^ k_swizzle<D>(row)) * 8) * 2u;
-    }
+    const uint32_t off = uint32_t(row * D + (ld_pch ^ bwd_swizzle<D>(row)) * 8) * 2u;
     buffer_to_lds_b128(rsrc, off, uint32_t(row0) * uint32_t(D * 2), lds_tile + uint32_t(w) * 1024u + uint32_t(i) * (NT * 16u));
   }
-}
-
-// A operand, row-wise: rows 32t + c of the tile, k-step s.
-template <int D>
-__device__ __forceinline__ u32x4_t bwd_row_frag(const uint16_t* tile, int s, int t, int g, int c) {
-  const int row = 32 * t + c;
-  const int ch = (2 * s + g) ^ k_swizzle<D>(row);
-  return *reinterpret_cast<const u32x4_t*>(tile + row * D + ch * 8);
-}
-// A operand, transposed: rows 32 dt .. +31 of tile^T at tile rows 16 ts .. +15, the 16 rows
-// taken in the accumulator order of the first product.
-template <int D>
-__device__ __forceinline__ u32x4_t bwd_tr_frag(const uint16_t* tile, int ts, int dt, int g, int c) {
-  const int i16 = c & 15, j16 = c >> 4;
-  const int vrow = 16 * ts + 4 * g + (i16 >> 2);
-  const int unit = 2 * dt + j16;
-  const int u0 = unit ^ v_swizzle<D>(vrow);
-  const int u1 = unit ^ v_swizzle<D>(vrow + 8);
-  const s16x4_t lo = lds_read_tr16(tile + vrow * D + u0 * 16 + (i16 & 3) * 4);
-  const s16x4_t hi = lds_read_tr16(tile + (vrow + 8) * D + u1 * 16 + (i16 & 3) * 4);
-  const u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo);
-  const u32x2_t hi2 = __builtin_bit_cast(u32x2_t, hi);
-  const u32x4_t a = {lo2[0], lo2[1], hi2[0], hi2[1]};
-  return a;
 }
 
 // 32 mask bytes -> 32 bits (any non-zero byte = 1), byte i -> bit i.
@@ -235,8 +214,8 @@ struct BwdDqTraits {
   static constexpr int kThreads = QB * 2;
   static constexpr int kStep = BwdRows<D, kThreads>::value;
   static constexpr int kTileElems = kStep * D;
-  // two sets of three tiles (K row-wise, K transposed, V row-wise), or the output staging
-  static constexpr size_t kLdsBytes = (6 * kTileElems > QB * D ? 6 * kTileElems : QB * D) * sizeof(uint16_t);
+  // two sets of two tiles (K, V), or the output staging
+  static constexpr size_t kLdsBytes = (4 * kTileElems > QB * D ? 4 * kTileElems : QB * D) * sizeof(uint16_t);
 };
 
 template <bool BF16, bool CAP, int D, int QB, int KB>
@@ -251,7 +230,7 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   constexpr int TILE = Traits::kTileElems;
 
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-  uint16_t* const lds16 = reinterpret_cast<uint16_t*>(lds_raw);  // [2 sets][Ka, Kt, Va][TILE]
+  uint16_t* const lds16 = reinterpret_cast<uint16_t*>(lds_raw);  // [2 sets][K, V][TILE]
 
   // Workgroup -> (slab, query block): XCD x takes the slabs bh with bh % n_xcd == x one after
   // the other, longest query block first, so the workgroups that run together on an XCD walk the
@@ -373,21 +352,20 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   };
   const uint32_t lds_tiles = lds_offset_of(lds16);
   auto issue_loads = [&](const BwdStepInfo& st, int set) {
-    const uint32_t base = lds_tiles + uint32_t(set) * (3u * TILE * 2u);
-    bwd_load_tile<D, NT, STEP, false>(rK, st.row0, base, tid, w);
-    bwd_load_tile<D, NT, STEP, true>(rK, st.row0, base + TILE * 2u, tid, w);
-    bwd_load_tile<D, NT, STEP, false>(rV, st.row0, base + 2u * TILE * 2u, tid, w);
+    const uint32_t base = lds_tiles + uint32_t(set) * (2u * TILE * 2u);
+    bwd_load_tile<D, NT, STEP>(rK, st.row0, base, tid, w);
+    bwd_load_tile<D, NT, STEP>(rV, st.row0, base + TILE * 2u, tid, w);
   };
   const uint32_t row_lane = bwd_row_lane<D>(g, c);
-  const uint32_t tr_lane = bwd_tr_lane<D>(g, c);
+  const uint32_t tr_lo = bwd_tr_lane<D>(g, c, 0), tr_hi = bwd_tr_lane<D>(g, c, 1);
   constexpr int PF = KS < 3 ? KS : 3;  // k-steps whose fragments are read ahead of their products
 
   // One step: S^T = K.Q^T and dP^T = V.dO^T (lane = query row, registers = keys), then
   // dS^T = P^T (dP^T - delta) packed to 16 bits in the order the next product reads it, then
   // dQ^T += K^T.dS^T.
   auto compute = [&](int set, const uint32_t (&kw)[NTL], bool all_allowed) {
-    const uint32_t base = lds_tiles + uint32_t(set) * (3u * TILE * 2u);
-    const uint32_t aK = base + row_lane, aV = aK + 2u * TILE * 2u, tK = base + TILE * 2u + tr_lane;
+    const uint32_t base = lds_tiles + uint32_t(set) * (2u * TILE * 2u);
+    const uint32_t aK = base + row_lane, aV = aK + TILE * 2u, tK0 = base + tr_lo, tK1 = base + tr_hi;
     f32x16_t st[NTL], dp[NTL];
     static_for<NTL>([&](auto tc) {
       constexpr int t = decltype(tc)::value;
@@ -413,7 +391,7 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
     u32x4_t ft[NTS][DT];  // fragments of the second product, read one 16-key group ahead
     static_for<DT>([&](auto dc) {
       constexpr int dt = decltype(dc)::value;
-      ft[0][dt] = lds_tr_pair_at(tK ^ uint32_t(64 * dt), 8u * D * 2u);
+      ft[0][dt] = lds_tr_pair_at(tK0 ^ uint32_t(64 * dt), tK1 ^ uint32_t(64 * dt));
     });
     __builtin_amdgcn_sched_barrier(0);
     u32x4_t dsb[NTL][2];
@@ -445,7 +423,8 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
       if constexpr (ts + 1 < NTS) {
         static_for<DT>([&](auto dc) {
           constexpr int dt = decltype(dc)::value;
-          ft[ts + 1][dt] = lds_tr_pair_at((tK ^ uint32_t(64 * dt)) + uint32_t(ts + 1) * 16u * D * 2u, 8u * D * 2u);
+          ft[ts + 1][dt] = lds_tr_pair_at((tK0 ^ uint32_t(64 * dt)) + uint32_t(ts + 1) * 16u * D * 2u,
+                                          (tK1 ^ uint32_t(64 * dt)) + uint32_t(ts + 1) * 16u * D * 2u);
         });
       }
       static_for<DT>([&](auto dc) {
@@ -509,15 +488,15 @@ struct BwdDkdvTraits {
   static constexpr int kStep = 32;                 // query rows per step
   static constexpr int kTileElems = kStep * D;
   static constexpr int kMaxBitmapWords = 4096;     // 64-slot words of the match bitmap
-  // two sets of four tiles (Q and dO, each row-wise and transposed; the output staging overlaps
-  // them); two sets of the weights one role hands to the other (fp32, [key group][16][64 lanes]);
-  // -delta and the exponent offsets of the rows of two steps; per 64-slot word of a slab's
-  // metadata the bitmap of the slots that list this KV block and mode / tile index of the first
-  static constexpr size_t kTileBytes = size_t(8) * kTileElems * sizeof(uint16_t);
+  // three sets of two tiles (Q, dO); two sets of the weights one role hands to the other (fp32,
+  // [key group][16][64 lanes]) -- the output staging overlaps tiles and weights; -delta and the
+  // exponent offsets of the rows of three steps; per 64-slot word of a slab's metadata the
+  // bitmap of the slots that list this KV block and mode / tile index of the first
+  static constexpr size_t kTileBytes = size_t(6) * kTileElems * sizeof(uint16_t);
   static constexpr size_t kWeightBytes = size_t(2) * kKeyGroups * 16 * 64 * sizeof(float);
   // (the launch asks for the words its metadata needs, so small problems fit two workgroups)
   static constexpr size_t lds_bytes(size_t bitmap_words) {
-    return kTileBytes + kWeightBytes + 4 * kStep * sizeof(float) + bitmap_words * (8 + 4);
+    return kTileBytes + kWeightBytes + 6 * kStep * sizeof(float) + bitmap_words * (8 + 4);
   }
   static constexpr size_t kLdsBytes = lds_bytes(kMaxBitmapWords);
 };
@@ -530,8 +509,8 @@ struct BwdDkdvTraits {
 //   the "gradient" wave holds V, computes dP - delta = dO.V^T - delta, and one step later
 //   dS = P (dP - delta) and dK^T += Q^T.dS.
 // The gradient waves run one step behind the weight waves, so one barrier per step orders
-// the hand-over, the tile loads (each role loads the two tiles it reads) and the reuse of the
-// two buffer sets.
+// the hand-over, the tile loads (the weight waves load Q, the gradient waves dO, one step ahead)
+// and the reuse of the three tile sets.
 template <bool BF16, bool CAP, int D, int QB, int KB>
 __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) {
   using Traits = BwdDkdvTraits<D, KB>;
@@ -547,11 +526,11 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
   constexpr int NTR = (STEP / 16) * DT;  // fragments of the second product
 
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-  uint16_t* const lds16 = reinterpret_cast<uint16_t*>(lds_raw);  // [2 sets][Qa, Qt, Da, Dt][TILE]
+  uint16_t* const lds16 = reinterpret_cast<uint16_t*>(lds_raw);  // [3 sets][Q, dO][TILE]
   float* const sW = reinterpret_cast<float*>(lds_raw + Traits::kTileBytes);  // [2 sets][NKG][16][64]
-  float* const sNd = sW + 2 * NKG * 16 * 64;                                 // [2 sets][STEP] -delta
-  float* const sL2 = sNd + 2 * STEP;                                         // [2 sets][STEP] exponent offsets
-  uint64_t* const sMatch = reinterpret_cast<uint64_t*>(sL2 + 2 * STEP);
+  float* const sNd = sW + 2 * NKG * 16 * 64;                                 // [3 sets][STEP] -delta
+  float* const sL2 = sNd + 3 * STEP;                                         // [3 sets][STEP] exponent offsets
+  uint64_t* const sMatch = reinterpret_cast<uint64_t*>(sL2 + 3 * STEP);
   int32_t* const sFirst = reinterpret_cast<int32_t*>(sMatch + p.Tq * ((p.max_blocks + 63) / 64));
 
   // Workgroup -> (slab, KV block): XCD x takes the slabs bh with bh % n_xcd == x one after the
@@ -679,27 +658,25 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
   const uint32_t lds_tiles = lds_offset_of(lds16);
   const uint32_t lds_w = lds_offset_of(sW) + uint32_t(kg) * 4096u + uint32_t(lane) * 16u;
   const uint32_t lds_nd = lds_offset_of(sNd), lds_l2 = lds_offset_of(sL2);
-  auto tile_at = [&](int set, int which) { return lds_tiles + uint32_t(set * 4 + which) * (TILE * 2u); };
-  // Each role loads what it reads: row-wise Q, transposed dO and the exponent offsets (weight
-  // waves); row-wise dO, transposed Q and -delta (gradient waves).
-  auto load_weight_tiles = [&](const BwdStepInfo& st, int set) {
-    bwd_load_tile<D, RT, STEP, false>(rQ, st.row0, tile_at(set, 0), rtid, kg);
-    bwd_load_tile<D, RT, STEP, true>(rD, st.row0, tile_at(set, 3), rtid, kg);
+  auto tile_at = [&](int set, int which) { return lds_tiles + uint32_t(set * 2 + which) * (TILE * 2u); };
+  // The rows of step j + 1 are loaded during iteration j: Q and the exponent offsets by the
+  // weight waves, dO and -delta by the gradient waves.
+  auto load_q = [&](const BwdStepInfo& st, int set) {
+    bwd_load_tile<D, RT, STEP>(rQ, st.row0, tile_at(set, 0), rtid, kg);
     if (rtid < STEP)
       buffer_to_lds_b32(rL2, uint32_t(rtid) * 4u, uint32_t(st.row0) * 4u, lds_l2 + uint32_t(set * STEP) * 4u);
   };
-  auto load_grad_tiles = [&](const BwdStepInfo& st, int set) {
-    bwd_load_tile<D, RT, STEP, false>(rD, st.row0, tile_at(set, 2), rtid, kg);
-    bwd_load_tile<D, RT, STEP, true>(rQ, st.row0, tile_at(set, 1), rtid, kg);
+  auto load_do = [&](const BwdStepInfo& st, int set) {
+    bwd_load_tile<D, RT, STEP>(rD, st.row0, tile_at(set, 1), rtid, kg);
     if (rtid < STEP)
       buffer_to_lds_b32(rNd, uint32_t(rtid) * 4u, uint32_t(st.row0) * 4u, lds_nd + uint32_t(set * STEP) * 4u);
   };
   const uint32_t row_lane = bwd_row_lane<D>(g, c);
-  const uint32_t tr_lane = bwd_tr_lane<D>(g, c);
+  const uint32_t tr_lo = bwd_tr_lane<D>(g, c, 0), tr_hi = bwd_tr_lane<D>(g, c, 1);
 
   // Weight wave, one step: S = Q.K^T (lane = key, registers = query rows), P, dV^T += dO^T.P.
-  auto weight_step = [&](int set, uint32_t kw, bool all_allowed) {
-    const uint32_t aQ = tile_at(set, 0) + row_lane, tD = tile_at(set, 3) + tr_lane;
+  auto weight_step = [&](int set, int par, uint32_t kw, bool all_allowed) {
+    const uint32_t aQ = tile_at(set, 0) + row_lane, tD0 = tile_at(set, 1) + tr_lo, tD1 = tile_at(set, 1) + tr_hi;
     u32x4_t fa[KS];
     static_for<KS>([&](auto ks) {
       constexpr int s = decltype(ks)::value;
@@ -714,7 +691,8 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
     u32x4_t gd[NTR];
     static_for<NTR>([&](auto jc) {
       constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
-      gd[ts * DT + dt] = lds_tr_pair_at((tD ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u, 8u * D * 2u);
+      gd[ts * DT + dt] = lds_tr_pair_at((tD0 ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u,
+                                        (tD1 ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u);
     });
     f32x4_t l4[4];
     static_for<4>([&](auto ic) {
@@ -738,7 +716,7 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
           pv[e] = wgt;
           hand[e] = wgt * fac;
         }
-        *(__attribute__((address_space(3))) f32x4_t*)(lds_w + uint32_t(set) * (NKG * 4096u) + uint32_t(i4) * 1024u) = hand;
+        *(__attribute__((address_space(3))) f32x4_t*)(lds_w + uint32_t(par) * (NKG * 4096u) + uint32_t(i4) * 1024u) = hand;
         pb[i4 >> 1][2 * (i4 & 1) + 0] = pack2<BF16>(pv[0], pv[1]);
         pb[i4 >> 1][2 * (i4 & 1) + 1] = pack2<BF16>(pv[2], pv[3]);
       });
@@ -755,8 +733,8 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
   };
   // Gradient wave, one step: dP - delta = dO.V^T - delta (the accumulator starts at -delta),
   // dS = P (dP - delta) with the partner's P, dK^T += Q^T.dS.
-  auto grad_step = [&](int set) {
-    const uint32_t aD = tile_at(set, 2) + row_lane, tQ = tile_at(set, 1) + tr_lane;
+  auto grad_step = [&](int set, int par) {
+    const uint32_t aD = tile_at(set, 1) + row_lane, tQ0 = tile_at(set, 0) + tr_lo, tQ1 = tile_at(set, 0) + tr_hi;
     f32x16_t dp;
     static_for<4>([&](auto ic) {
       constexpr int i4 = decltype(ic)::value;
@@ -779,12 +757,13 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
     u32x4_t gq[NTR];
     static_for<NTR>([&](auto jc) {
       constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
-      gq[ts * DT + dt] = lds_tr_pair_at((tQ ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u, 8u * D * 2u);
+      gq[ts * DT + dt] = lds_tr_pair_at((tQ0 ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u,
+                                        (tQ1 ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u);
     });
     f32x4_t hand[4];
     static_for<4>([&](auto ic) {
       constexpr int i4 = decltype(ic)::value;
-      hand[i4] = lds_f32x4_at(lds_w + uint32_t(set) * (NKG * 4096u) + uint32_t(i4) * 1024u);
+      hand[i4] = lds_f32x4_at(lds_w + uint32_t(par) * (NKG * 4096u) + uint32_t(i4) * 1024u);
     });
     __builtin_amdgcn_sched_barrier(0);
     u32x4_t dsb[2];
@@ -827,8 +806,9 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
     constexpr bool GRAD = decltype(role_c)::value;
     const BwdStepInfo none = {0, kMasked, -1, 0, 0, false};
     BwdStepInfo prev = none, cur = next_step();
-    if constexpr (!GRAD) {
-      if (cur.valid) load_weight_tiles(cur, 0);
+    int s_prev = 2, s_cur = 0, s_nxt = 1;  // tile sets of steps j - 1, j, j + 1
+    if (cur.valid) {
+      if constexpr (!GRAD) load_q(cur, 0); else load_do(cur, 0);
     }
     for (int j = 0; cur.valid || prev.valid; ++j) {
       const BwdStepInfo nxt = cur.valid ? next_step() : none;
@@ -845,18 +825,22 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
           kw = m >> (4 * g);
         }
       }
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the tiles this wave loaded have landed
-      __syncthreads();  // ... everybody's have; the hand-over of step j - 1 is written; the sets
-                        // about to be overwritten are no longer read
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the tile this wave loaded has landed
+      __syncthreads();  // ... everybody's have; the hand-over of step j - 1 is written; the set
+                        // about to be overwritten (step j - 2) is no longer read
       if constexpr (!GRAD) {
-        if (nxt.valid) load_weight_tiles(nxt, (j + 1) & 1);
-        if (cur.valid) weight_step(j & 1, kw, cur.mode == kFull && key_wave_min + 32 <= p.seqlen);
+        if (nxt.valid) load_q(nxt, s_nxt);
+        if (cur.valid) weight_step(s_cur, j & 1, kw, cur.mode == kFull && key_wave_min + 32 <= p.seqlen);
       } else {
-        if (cur.valid) load_grad_tiles(cur, j & 1);
-        if (prev.valid) grad_step((j + 1) & 1);
+        if (nxt.valid) load_do(nxt, s_nxt);
+        if (prev.valid) grad_step(s_prev, (j + 1) & 1);
       }
       prev = cur;
       cur = nxt;
+      const int t3 = s_prev;
+      s_prev = s_cur;
+      s_cur = s_nxt;
+      s_nxt = t3;
     }
     __syncthreads();
     uint16_t* stage = lds16 + size_t(w) * 32 * D;
