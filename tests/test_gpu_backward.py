@@ -14,7 +14,7 @@ import torch
 import omni_attn_capi
 from baseline_configs import make_workload
 from helpers import random_block_metadata
-from oracle.dense_oracle import attention_dense_grads, dense_mask_from_blocks, prefix_mask
+from oracle.dense_oracle import attention_dense_fp32, attention_dense_grads, dense_mask_from_blocks, prefix_mask
 
 pytestmark = pytest.mark.gpu
 
@@ -89,6 +89,44 @@ def test_random_metadata_backward(dtype, D, QB, KB, gpu_device):
         check_grads(got[:3], ref, dtype, f"random metadata seqlen={seqlen}")
         for t in got[:3]:
             assert (t[:, :, seqlen:] == 0).all(), "rows beyond the sequence must get zero gradients"
+
+
+def test_wide_block_lists_backward(gpu_device):
+    """Lists wider than 64 and 128 slots (most of them MASKED padding, the real blocks scattered over
+    the whole width): the metadata of a query block then spans several 64-slot words, in the dQ
+    kernel's register chunks and in the dK/dV kernel's match bitmap alike."""
+    gen = torch.Generator().manual_seed(105)
+    B, H, S, D, QB, KB, W = 1, 2, 512, 64, 128, 64, 150
+    Tq, Tk = S // QB, S // KB
+    q, k, v, dout = (torch.randn(B, H, S, D, generator=gen).to(torch.float16) for _ in range(4))
+    nb = torch.zeros(B, H, Tq, dtype=torch.int32)
+    idx = torch.randint(0, Tk, (B, H, Tq, W), generator=gen, dtype=torch.int32)
+    tys = torch.zeros(B, H, Tq, W, dtype=torch.int32)  # MASKED
+    pidx = torch.full((B, H, Tq, W), -1, dtype=torch.int32)
+    tiles = []
+    for h in range(H):
+        for qb in range(Tq):
+            cols = [kb for kb in range(Tk) if torch.rand((), generator=gen).item() > 0.25]
+            slots = sorted(torch.randperm(W, generator=gen)[:len(cols)].tolist())
+            if qb == 1:
+                slots[-1] = W - 1  # the last slot of the list
+            if qb == 2 and len(slots) > 1:
+                slots[0], slots[1] = 63, 64  # either side of a word boundary
+            nb[0, h, qb] = W if qb != 3 else slots[-1] + 1
+            for s, kb in zip(slots, cols):
+                idx[0, h, qb, s] = kb
+                ty = (2, 1, 3)[int(torch.randint(0, 3, (), generator=gen))]
+                tys[0, h, qb, s] = ty
+                if ty == 3:
+                    pidx[0, h, qb, s] = len(tiles)
+                    tiles.append(torch.rand(QB, KB, generator=gen) < 0.5)
+    pm = torch.stack(tiles).to(torch.uint8)
+    got = run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, S, pidx, pm, device=gpu_device)
+    dense = dense_mask_from_blocks(nb, idx, tys, QB, KB, S, S, pidx, pm, seqlen_orig=S)
+    ref = attention_dense_grads(q, k, v, dense, dout)
+    check_grads(got[:3], ref, torch.float16, "wide lists")
+    fwd_ref, _ = attention_dense_fp32(q, k, v, dense)
+    assert (got[3].float().cpu() - fwd_ref).abs().max().item() <= 2e-3
 
 
 def test_c2_full_size_backward_on_sampled_slabs(gpu_device):

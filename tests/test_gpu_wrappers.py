@@ -82,9 +82,16 @@ def test_module_errors_on_gpu_tensors(gpu_device):
     with pytest.raises(RuntimeError, match="torch.bool"):
         omni_attn.omni_attn_simple_kernel(q, q, q, q.clone(), nb, idx, idx, 128, 128, 256, idx,
                                           torch.zeros(1, 128, 128, dtype=torch.uint8, device=gpu_device), True)
+    # the matrix-core entry points take head_dim 32 / 64 / 128 only; the simple one (scalar-semantics
+    # kernel behind it) any head_dim up to 256
     q96 = torch.zeros(1, 2, 256, 96, dtype=torch.float16, device=gpu_device)
     with pytest.raises(RuntimeError, match="head_dim"):
-        omni_attn.omni_attn_simple_kernel(q96, q96, q96, q96.clone(), nb, idx, idx, 128, 128, 256, e_i, e_b, False)
+        omni_attn.omni_attn_cp_async(q96, q96, q96, q96.clone(), nb, idx, idx, 128, 128, 256, e_i, e_b, False)
+    omni_attn.omni_attn_simple_kernel(q96, q96, q96, q96.clone(), nb, idx, torch.full_like(idx, 2), 128, 128, 256,
+                                      e_i, e_b, False)
+    q264 = torch.zeros(1, 2, 256, 264, dtype=torch.float16, device=gpu_device)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        omni_attn.omni_attn_simple_kernel(q264, q264, q264, q264.clone(), nb, idx, idx, 128, 128, 256, e_i, e_b, False)
     # and a good call still works afterwards
     omni_attn.omni_attn_simple_kernel(q, q, q, q.clone(), nb, idx, torch.full_like(idx, 2), 128, 128, 256, e_i, e_b, False)
     torch.cuda.synchronize()
