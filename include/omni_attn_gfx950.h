@@ -175,8 +175,9 @@ int omni_attn_fwd_packed_gfx950(const void* q, const void* k, const void* v, voi
  *   partial tiles     as bytes (partial_masks_or_null) or packed (partial_bits_or_null);
  *                     pass one of them or neither.
  *   workspace         device memory of at least omni_attn_bwd_workspace_bytes(B, H, S_pad)
- *                     bytes, 4-byte aligned; holds rowsum(dout . o) between the two kernels
- *                     of the backward.  Contents before and after the call are meaningless.
+ *                     bytes (two floats per row), 4-byte aligned; holds -rowsum(dout . o) and
+ *                     the rows' exponent offsets between the two kernels of the backward.
+ *                     Contents before and after the call are meaningless.
  * Limits beyond the forward's: Tq * ceil(max_blocks / 64) <= 4096 (OMNI_ATTN_ERR_TOO_LARGE).
  * Two kernels are enqueued on `stream`; nothing is allocated; results are bitwise reproducible.
  */

@@ -367,6 +367,7 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
     const uint32_t base = lds_tiles + uint32_t(set) * (2u * TILE * 2u);
     const uint32_t aK = base + row_lane, aV = aK + TILE * 2u, tK0 = base + tr_lo, tK1 = base + tr_hi;
     f32x16_t st[NTL], dp[NTL];
+    __builtin_amdgcn_s_setprio(1);  // products first: the other wave of the SIMD fills the gaps
     static_for<NTL>([&](auto tc) {
       constexpr int t = decltype(tc)::value;
       constexpr uint32_t trow = uint32_t(t) * 32u * D * 2u;
@@ -393,6 +394,7 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
       constexpr int dt = decltype(dc)::value;
       ft[0][dt] = lds_tr_pair_at(tK0 ^ uint32_t(64 * dt), tK1 ^ uint32_t(64 * dt));
     });
+    __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
     u32x4_t dsb[NTL][2];
     auto weights = [&](auto masked_c) {
@@ -418,6 +420,7 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
     } else {
       weights(std::integral_constant<bool, true>{});
     }
+    __builtin_amdgcn_s_setprio(1);
     static_for<NTS>([&](auto tsc) {
       constexpr int ts = decltype(tsc)::value;
       if constexpr (ts + 1 < NTS) {
@@ -433,6 +436,7 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
       });
       __builtin_amdgcn_sched_barrier(0);
     });
+    __builtin_amdgcn_s_setprio(0);
   };
 
   // Tiles of step i + 1 are loaded while step i is computed: one barrier per step.
@@ -683,11 +687,13 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
       fa[s] = lds_b128_at(aQ ^ uint32_t(32 * s));
     });
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(1);  // products first (it pays with two workgroups per compute unit)
     f32x16_t sc = zero16;
     static_for<KS>([&](auto ks) {
       constexpr int s = decltype(ks)::value;
       sc = mfma_32x32x16<BF16>(fa[s], bop[s], sc);
     });
+    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(0);
     u32x4_t gd[NTR];
     static_for<NTR>([&](auto jc) {
       constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
@@ -726,10 +732,12 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
     } else {
       weights(std::integral_constant<bool, true>{});
     }
+    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(1);
     static_for<NTR>([&](auto jc) {
       constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
       acc[dt] = mfma_32x32x16<BF16>(gd[ts * DT + dt], pb[ts], acc[dt]);
     });
+    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(0);
   };
   // Gradient wave, one step: dP - delta = dO.V^T - delta (the accumulator starts at -delta),
   // dS = P (dP - delta) with the partner's P, dK^T += Q^T.dS.
@@ -750,10 +758,12 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
       fb[s] = lds_b128_at(aD ^ uint32_t(32 * s));
     });
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(1);
     static_for<KS>([&](auto ks) {
       constexpr int s = decltype(ks)::value;
       dp = mfma_32x32x16<BF16>(fb[s], bop[s], dp);
     });
+    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(0);
     u32x4_t gq[NTR];
     static_for<NTR>([&](auto jc) {
       constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
@@ -772,10 +782,12 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
       dsb[i4 >> 1][2 * (i4 & 1) + 0] = pack2<BF16>(hand[i4][0] * dp[4 * i4 + 0], hand[i4][1] * dp[4 * i4 + 1]);
       dsb[i4 >> 1][2 * (i4 & 1) + 1] = pack2<BF16>(hand[i4][2] * dp[4 * i4 + 2], hand[i4][3] * dp[4 * i4 + 3]);
     });
+    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(1);
     static_for<NTR>([&](auto jc) {
       constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
       acc[dt] = mfma_32x32x16<BF16>(gq[ts * DT + dt], dsb[ts], acc[dt]);
     });
+    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(0);
   };
 
   // Bits of one partial tile for this lane's key: bit j = query row q_local0 + j of the tile

@@ -77,6 +77,47 @@ class OmniBlockMask:
                 self.partial_block_masks.to(torch.bool).contiguous())
         return self
 
+    def deduplicate_partial_tiles(self) -> "OmniBlockMask":
+        """Keep one copy of every distinct PARTIAL tile and point the slots at it.
+
+        The reference stores a tile per (batch, head, q_block, slot) in visiting order
+        (omni_attn_torch.py:173-196), so a mask that is the same for every head holds H copies of
+        each tile.  The kernels only follow ``partial_block_mask_indices``; sharing tiles changes
+        no result.  Kept tiles stay in order of first appearance.  Runs where the mask lives."""
+        pm = self.partial_block_masks
+        if pm is None or self.partial_block_mask_indices is None or pm.shape[0] < 2:
+            return self
+        P = pm.shape[0]
+        dev = pm.device
+        if self.partial_block_bits is not None:
+            rows = self.partial_block_bits.reshape(P, -1)
+        else:  # 8 mask bytes -> one byte of bits, so the sort behind unique() moves 8x less
+            flat = (pm.reshape(P, -1) != 0).to(torch.uint8)
+            pad = (-flat.shape[1]) % 8
+            if pad:
+                flat = torch.nn.functional.pad(flat, (0, pad))
+            weights = (2 ** torch.arange(8, device=dev, dtype=torch.int32)).view(1, 1, 8)
+            rows = (flat.view(P, -1, 8).to(torch.int32) * weights).sum(-1).to(torch.uint8)
+        uniq, inverse = torch.unique(rows, dim=0, return_inverse=True)
+        U = uniq.shape[0]
+        if U == P:
+            return self
+        first = torch.full((U,), P, dtype=torch.long, device=dev)
+        first.scatter_reduce_(0, inverse, torch.arange(P, device=dev), reduce="amin")
+        order = torch.argsort(first)                      # unique tiles by first appearance
+        rank = torch.empty_like(order)
+        rank[order] = torch.arange(U, device=dev)
+        new_id = rank[inverse].to(torch.int32)            # old tile number -> new tile number
+        keep = first[order]
+        old = self.partial_block_mask_indices
+        safe = old.clamp(min=0, max=P - 1).long()
+        valid = (old >= 0) & (old < P)
+        self.partial_block_mask_indices = torch.where(valid, new_id.to(old.device)[safe], old)
+        self.partial_block_masks = pm[keep].contiguous()
+        if self.partial_block_bits is not None:
+            self.partial_block_bits = self.partial_block_bits[keep].contiguous()
+        return self
+
     @property
     def num_q_blocks(self) -> int:
         return (self.q_len + self.Q_BLOCK_SIZE - 1) // self.Q_BLOCK_SIZE

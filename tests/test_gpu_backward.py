@@ -91,6 +91,21 @@ def test_random_metadata_backward(dtype, D, QB, KB, gpu_device):
             assert (t[:, :, seqlen:] == 0).all(), "rows beyond the sequence must get zero gradients"
 
 
+def test_slab_counts_that_do_not_divide_over_the_xcds(gpu_device):
+    """15 and 9 slabs: the kernels deal slabs to the 8 XCDs round-robin, so some XCDs get one slab
+    more than others (forward and backward)."""
+    for B, H in ((3, 5), (1, 9)):
+        gen = torch.Generator().manual_seed(106 + B)
+        S, D, QB, KB = 384, 64, 128, 128
+        q, k, v, dout = (torch.randn(B, H, S, D, generator=gen).to(torch.bfloat16) for _ in range(4))
+        nb, idx, tys, pidx, pm = random_block_metadata(gen, B, H, S // QB, S // KB, QB, KB, shuffle=True)
+        got = run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, S - 7, pidx, pm, device=gpu_device)
+        dense = dense_mask_from_blocks(nb, idx, tys, QB, KB, S, S, pidx, pm, seqlen_orig=S - 7)
+        check_grads(got[:3], attention_dense_grads(q, k, v, dense, dout), torch.bfloat16, f"{B * H} slabs")
+        fwd_ref, _ = attention_dense_fp32(q, k, v, dense)
+        assert (got[3].float().cpu() - fwd_ref).abs().max().item() <= 1e-2
+
+
 def test_wide_block_lists_backward(gpu_device):
     """Lists wider than 64 and 128 slots (most of them MASKED padding, the real blocks scattered over
     the whole width): the metadata of a query block then spans several 64-slot words, in the dQ

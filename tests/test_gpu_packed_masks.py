@@ -118,3 +118,27 @@ def test_wrappers_use_packed_tiles_when_the_mask_has_them(gpu_device):
     assert torch.equal(o_bits, o_bytes) and torch.equal(lse_bits, lse_bytes) and torch.equal(o_sw, o_bytes)
     ro, rl = attention_dense_fp32(w.q, w.k, w.v, prefix_mask(w.prefix_len, 1024).unsqueeze(1))
     compare_with_oracle(o_bits, lse_bits, ro, rl, w.dtype, "wrapper on packed tiles")
+
+
+def test_deduplicated_tiles_give_the_same_output(gpu_device):
+    """Sharing equal PARTIAL tiles between heads (on the GPU, on bytes and on packed words) leaves
+    the forward bit for bit the same."""
+    import omni_attn_torch as oat
+    gen = torch.Generator().manual_seed(12)
+    B, H, S, D = 1, 4, 512, 64
+    dense = (torch.rand(B, 1, S, S, generator=gen) < 0.6).expand(B, H, S, S).contiguous()
+    dense[..., torch.arange(S), torch.arange(S)] = True
+    q, k, v = (torch.randn(B, H, S, D, generator=gen).half().to(gpu_device) for _ in range(3))
+    m = oat.create_omni_block_mask_from_dense(dense, 128, 128).to(gpu_device)
+    P = m.partial_block_masks.shape[0]
+    o_ref, lse_ref = oat.omni_attention_forward(q, k, v, m)
+    m_bytes = oat.create_omni_block_mask_from_dense(dense, 128, 128).to(gpu_device).deduplicate_partial_tiles()
+    m_bits = oat.create_omni_block_mask_from_dense(dense, 128, 128).to(gpu_device).pack_partial_masks()
+    m_bits.deduplicate_partial_tiles()
+    for mm in (m_bytes, m_bits):
+        assert mm.partial_block_masks.shape[0] == P // H and mm.partial_block_masks.is_cuda
+        o, lse = oat.omni_attention_forward(q, k, v, mm)
+        assert torch.equal(o, o_ref) and torch.equal(lse, lse_ref)
+    assert m_bits.partial_block_bits.shape[0] == P // H
+    ro, rl = attention_dense_fp32(q.cpu(), k.cpu(), v.cpu(), dense)
+    compare_with_oracle(o_ref, lse_ref, ro, rl, torch.float16, "de-duplicated tiles")

@@ -131,6 +131,39 @@ def test_build_partial_block_data_matches_loops():
     assert tiles.shape == (count, QB, KB) and tiles.dtype == torch.bool and pidx.dtype == torch.int32
 
 
+def test_deduplicate_partial_tiles_shares_tiles_between_heads():
+    """A dense mask that is the same for every head: the reference's tile store holds one copy
+    per head (omni_attn_torch.py:173-196); after de-duplication one copy per distinct tile is
+    left, in order of first appearance, and the mask represents the same dense mask."""
+    gen = torch.Generator().manual_seed(11)
+    B, H, S, QB, KB = 2, 4, 512, 128, 64
+    per_batch = torch.rand(B, 1, S, S, generator=gen) < 0.5
+    per_batch[0, 0, :128, :64] = per_batch[0, 0, 128:256, 64:128]  # two equal tiles inside one head as well
+    dense = per_batch.expand(B, H, S, S).contiguous()
+    mask = create_omni_block_mask_from_dense(dense, QB, KB)
+    P = mask.partial_block_masks.shape[0]
+    assert P == B * H * (S // QB) * (S // KB)          # every tile is PARTIAL and stored per head
+    before = mask.to_dense_mask()
+    old_idx, old_tiles = mask.partial_block_mask_indices.clone(), mask.partial_block_masks.clone()
+    mask.deduplicate_partial_tiles()
+    U = mask.partial_block_masks.shape[0]
+    assert U == B * (S // QB) * (S // KB) - 1
+    assert torch.equal(mask.to_dense_mask(), before) and torch.equal(before, dense)
+    new_idx = mask.partial_block_mask_indices
+    assert new_idx.dtype == torch.int32 and torch.equal(new_idx < 0, old_idx < 0)
+    sel = old_idx >= 0
+    assert torch.equal(mask.partial_block_masks[new_idx[sel].long()], old_tiles[old_idx[sel].long()])
+    # order of first appearance: the tile numbers, in visiting order, never jump ahead
+    seq = new_idx[sel].tolist()
+    seen = -1
+    for t in seq:
+        assert t <= seen + 1
+        seen = max(seen, t)
+    # nothing to do the second time; masks without tiles pass through
+    assert mask.deduplicate_partial_tiles().partial_block_masks.shape[0] == U
+    assert create_causal_omni_block_mask(1, 2, 256, 256, device="cpu").deduplicate_partial_tiles().partial_block_masks is None
+
+
 def test_to_dense_mask_partial_fallbacks():
     """PARTIAL without stored bits: causal in the reference's to_dense_mask, skipped by the kernels."""
     nb = torch.tensor([[[1, 2]]], dtype=torch.int32)
