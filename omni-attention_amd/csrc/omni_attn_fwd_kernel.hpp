@@ -639,6 +639,11 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
       }
     };
 
+    // The slots run at a raised wave priority and everything between two bodies (barrier, rescale,
+    // mask, metadata of the next steps) at the default one: the other wave of the SIMD, from the
+    // other workgroup of the compute unit, is then not held up by this wave's bookkeeping while
+    // it has matrix instructions to issue.
+    __builtin_amdgcn_s_setprio(1);
     static_for<NS>([&](auto jc) {
       constexpr int j = decltype(jc)::value;
       if constexpr (j < NPV) {
@@ -654,6 +659,7 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
       static_for<u_hi - u_lo>([&](auto dc) { vector_chunk(IntC<u_lo + decltype(dc)::value>{}); });
       __builtin_amdgcn_sched_barrier(0);
     });
+    __builtin_amdgcn_s_setprio(0);
   };
 
   // ---- the walk -------------------------------------------------------------------------
