@@ -46,10 +46,11 @@ RESOURCES_JSON = os.path.join(OBJ, "kernel_resources.json")
 
 # What the kernels of the library must keep: no scratch memory, no spilled registers, and at
 # least this many waves per SIMD (kernels are matched by a substring of their mangled name).
-# The backward kernels are the plain schedule (one wave per SIMD, registers spilling into the
-# accumulation file, a few instances into scratch): they are recorded, not gated.
-MIN_WAVES_PER_SIMD = {"fwd_kernel": 2}
-NOT_GATED = ("bwd_dq_kernel", "bwd_dkdv_kernel", "fwd_generic_kernel")
+# The backward kernels keep scalar values in spare vector lanes here and there (SGPR spills, no
+# memory behind them): for them only scratch memory and spilled vector registers fail the build.
+MIN_WAVES_PER_SIMD = {"fwd_kernel": 2, "bwd_dq_kernel": 2}
+SGPR_SPILLS_ALLOWED = ("bwd_dq_kernel", "bwd_dkdv_kernel")
+NOT_GATED = ("fwd_generic_kernel",)
 
 INSTANCES = [(bf, d) for bf in (0, 1) for d in (32, 64, 128)]
 LIB_NAME = "libomni_attn_gfx950.so"
@@ -83,7 +84,8 @@ def check_resources(kernels):
     for name, r in sorted(kernels.items()):
         if any(tag in name for tag in NOT_GATED):
             continue
-        if r.get("scratch_bytes", 0) or r.get("vgpr_spills", 0) or r.get("sgpr_spills", 0):
+        sgpr_spills = 0 if any(tag in name for tag in SGPR_SPILLS_ALLOWED) else r.get("sgpr_spills", 0)
+        if r.get("scratch_bytes", 0) or r.get("vgpr_spills", 0) or sgpr_spills:
             problems.append("%s: scratch %d B/lane, %d VGPR / %d SGPR spills" % (
                 name, r.get("scratch_bytes", 0), r.get("vgpr_spills", 0), r.get("sgpr_spills", 0)))
         for pattern, waves in MIN_WAVES_PER_SIMD.items():

@@ -13,18 +13,22 @@
 //
 // Two kernels, no atomics, bitwise reproducible:
 //   bwd_dq_kernel    one workgroup per query block; walks that block's list like the forward;
-//                    also writes delta for its rows (workspace, read by the second kernel).
+//                    also writes -delta and the rows' exponent offsets (workspace, read by the
+//                    second kernel).
 //   bwd_dkdv_kernel  one workgroup per KV block; finds the (query block, slot) pairs that list
 //                    it by scanning the slab's metadata (a bitmap of the matches is built in
-//                    LDS first, then visited in ascending order).
-// The dQ kernel runs two workgroups per compute unit (two waves per SIMD, each hides the other's
-// loads); the dK/dV kernel needs more than 256 registers per lane and runs one.
+//                    LDS first, then visited in ascending order).  Each 32 keys have two waves
+//                    with different work (weights and dV / dP, dS and dK), so two waves share
+//                    a SIMD.
 // Both use the forward's building blocks with the operands exchanged: every product is a
-// v_mfma_f32_32x32x16 whose A operand comes from an LDS tile (row-wise or transposed read)
-// and whose B operand is in registers, and the accumulator of the first product of a step is
-// the B operand of the second one, so P and dS never leave registers.
-// Tiles are double-buffered (the loads of step i + 1 run under the products of step i, one barrier
-// per step); inside a step the products and the vector work are left to the compiler's schedule.
+// v_mfma_f32_32x32x16 whose A operand comes from an LDS tile (row-wise or transposed read of
+// the same tile) and whose B operand is in registers, and the accumulator of the first product
+// of a step is the B operand of the second one, so P and dS never leave registers (the dK/dV
+// kernel hands P from one wave to its partner through LDS).
+// Tiles are loaded one step ahead (one barrier per step) and the fragments of a product are read
+// ahead of it; inside a step the order of the products and the vector work is pinned, the rest
+// is the compiler's schedule.  Workgroups are dealt to the XCDs by slab, so the workgroups that
+// run together on an XCD share their operands through its L2.
 #pragma once
 
 #include "omni_attn_fwd_kernel.hpp"
