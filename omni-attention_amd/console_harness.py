@@ -16,6 +16,12 @@ Differences from the reference script:
     python omni-attention_amd/console_harness.py --workload c1_causal
     python omni-attention_amd/console_harness.py --save-fixture /tmp/c1.safetensors --workload c1_causal
     python omni-attention_amd/console_harness.py --fixture /tmp/c1.safetensors
+
+Per-kernel times from the profiler, for the same run:
+
+    rocprofv3 --kernel-trace --stats --output-format csv -d /tmp/prof -o run \
+        -- python3 omni-attention_amd/console_harness.py --workload c2_interleaved
+    python omni-attention_amd/console_harness.py --rocprof-summary /tmp/prof
 """
 import argparse
 import os
@@ -129,6 +135,33 @@ def run(q, k, v, block_mask: OmniBlockMask, device="cuda:0", warmup=3, iters=10,
     return results
 
 
+def rocprof_summary(path, out=sys.stdout, top=12):
+    """Print the per-kernel table of a `rocprofv3 --kernel-trace --stats --output-format csv` run:
+    ``path`` is a `*_kernel_stats.csv` file or a directory that holds some (searched recursively).
+    Returns the rows as (name, calls, average microseconds, percent of the traced kernel time)."""
+    import csv
+    import glob
+
+    files = [path] if os.path.isfile(path) else sorted(
+        glob.glob(os.path.join(path, "**", "*kernel_stats.csv"), recursive=True))
+    if not files:
+        raise FileNotFoundError(f"no *_kernel_stats.csv under {path}")
+    rows = []
+    for f in files:
+        with open(f, newline="") as fh:
+            for r in csv.DictReader(fh):
+                rows.append((r["Name"], int(r["Calls"]), float(r["AverageNs"]) * 1e-3, float(r["TotalDurationNs"])))
+    total = sum(r[3] for r in rows) or 1.0
+    rows.sort(key=lambda r: -r[3])
+    print(f"rocprofv3 kernel summary ({len(files)} file(s), {sum(r[1] for r in rows)} dispatches):", file=out)
+    result = []
+    for name, calls, avg_us, tot in rows[:top]:
+        short = name if len(name) <= 72 else name[:69] + "..."
+        print(f"  {100.0 * tot / total:6.2f}%  {calls:7d} x {avg_us:10.1f} us  {short}", file=out)
+        result.append((name, calls, avg_us, 100.0 * tot / total))
+    return result
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--workload", default="c1_causal")
@@ -136,7 +169,13 @@ def main(argv=None):
     ap.add_argument("--fixture", help="safetensors fixture to run instead of a workload")
     ap.add_argument("--save-fixture", help="write the workload as a safetensors fixture and exit")
     ap.add_argument("--iters", type=int, default=10)
+    ap.add_argument("--rocprof-summary", metavar="PATH",
+                    help="print the per-kernel table of a rocprofv3 --kernel-trace --stats csv run and exit")
     args = ap.parse_args(argv)
+
+    if args.rocprof_summary:
+        rocprof_summary(args.rocprof_summary)
+        return 0
 
     if args.fixture:
         q, k, v, m, _ = load_fixture(args.fixture)

@@ -23,6 +23,24 @@ def test_fixture_round_trip(tmp_path):
     assert torch.equal(m.to_dense_mask(), a.to_dense_mask())
 
 
+def test_rocprof_summary_reads_kernel_stats(tmp_path):
+    d = tmp_path / "prof" / "host" / "123"
+    d.mkdir(parents=True)
+    (d / "run_kernel_stats.csv").write_text(
+        '"Name","Calls","TotalDurationNs","AverageNs","Percentage","MinNs","MaxNs","StdDev"\n'
+        '"void omni_attn::fwd_kernel<true, 128, 128, 128>(omni_attn::FwdParams)",65,19500000,300000.0,97.5,290000,420000,9000.0\n'
+        '"void at::native::vectorized_elementwise_kernel<4, at::native::FillFunctor<float>, std::array<char*, 1ul> >(int, at::native::FillFunctor<float>, std::array<char*, 1ul>)",5,500000,100000.0,2.5,90000,110000,10.0\n')
+    buf = io.StringIO()
+    rows = console_harness.rocprof_summary(str(tmp_path / "prof"), out=buf)
+    assert rows[0][0].startswith("void omni_attn::fwd_kernel") and rows[0][1] == 65
+    assert abs(rows[0][2] - 300.0) < 1e-9 and abs(rows[0][3] - 97.5) < 1e-9 and abs(rows[1][3] - 2.5) < 1e-9
+    text = buf.getvalue()
+    assert "70 dispatches" in text and " 97.50%" in text and "300.0 us" in text
+    with pytest.raises(FileNotFoundError):
+        console_harness.rocprof_summary(str(tmp_path / "nothing"))
+    assert console_harness.main(["--rocprof-summary", str(d / "run_kernel_stats.csv")]) == 0
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("name,kw", [("c1_causal", {}), ("c3_partial", {"H": 2, "S": 1024})])
 def test_all_entry_points_pass_on_the_console(name, kw, gpu_device):
