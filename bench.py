@@ -291,8 +291,9 @@ def fixed_cost_study(dev, seed, steps, warmup):
             "rows": rows}
 
 
-def extra_workload(name, seed, dev, steps, warmup):
-    """Kernel time of another workload (HIP events on the launch stream, clock already settled)."""
+def extra_workload(name, seed, dev, steps, warmup, backward=False):
+    """Kernel time of another workload, or of the backward of a workload (HIP events on the launch
+    stream, clock already settled)."""
     import torch
 
     import omni_attn_capi
@@ -313,6 +314,18 @@ def extra_workload(name, seed, dev, steps, warmup):
         omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, pidx, pm,
                            stream=stream.cuda_stream)
 
+    if backward:
+        step()
+        g = torch.Generator(device="cpu").manual_seed(seed + 1)
+        dout = torch.randn(w.q.shape, generator=g).to(w.dtype).to(dev)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+        ws = torch.empty(omni_attn_capi.load_library().omni_attn_bwd_workspace_bytes(B, H, S), dtype=torch.uint8,
+                         device=dev)
+
+        def step():  # noqa: F811
+            omni_attn_capi.bwd(q, k, v, o, dout, lse, dq, dk, dv, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE,
+                               S, pidx, pm, None, workspace=ws, stream=stream.cuda_stream)
+
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -324,9 +337,12 @@ def extra_workload(name, seed, dev, steps, warmup):
         ends[i].record(stream)
     torch.cuda.synchronize()
     ms = sum(a.elapsed_time(b) for a, b in zip(starts, ends)) / steps
-    tf = w.effective_flops / (ms * 1e-3) / 1e12
-    return {"workload": f"{name}: B={B} H={H} S={S} D={D}", "nonempty_blocks": w.nonempty_blocks,
-            "kernel_ms_avg": ms, "tflops": tf, "frac": tf / MFMA_PEAK_TFLOPS}
+    tf = w.effective_flops * (2.5 if backward else 1.0) / (ms * 1e-3) / 1e12
+    out = {"workload": f"{name}: B={B} H={H} S={S} D={D}", "nonempty_blocks": w.nonempty_blocks,
+           "kernel_ms_avg": ms, "tflops": tf, "frac": tf / MFMA_PEAK_TFLOPS}
+    if backward:
+        out["pass"] = "backward (dQ kernel + dK/dV kernel), 10*QB*KB*D flop per listed block"
+    return out
 
 
 def main(argv=None):
@@ -338,7 +354,7 @@ def main(argv=None):
                     help="keep the GPU under the benchmark's own load for this long before the warm-up "
                          "launches (from idle the shader clock needs some tens of milliseconds to settle)")
     ap.add_argument("--no-extras", action="store_true",
-                    help="skip the measured MFMA peak and the c2_interleaved_8k figure")
+                    help="skip the measured MFMA peak, the c2_interleaved_8k figure and the backward figure")
     ap.add_argument("--kernel-source-hash", action="store_true", help="print the hash and exit")
     ap.add_argument("--backward", action="store_true",
                     help="time the backward (dQ kernel + dK/dV kernel) instead of the forward; effective "
@@ -532,6 +548,9 @@ def main(argv=None):
         if args.workload == "c2_interleaved":
             out["c2_interleaved_8k"] = extra_workload("c2_interleaved_8k", args.seed, dev, steps=args.steps,
                                                       warmup=max(args.warmup, 5))
+            if not args.backward:
+                out["c2_interleaved_backward"] = extra_workload("c2_interleaved", args.seed, dev,
+                                                                steps=min(args.steps, 50), warmup=5, backward=True)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, args.cpu_budget_s)
     print(json.dumps(out))
