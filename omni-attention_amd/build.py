@@ -40,6 +40,9 @@ DEVICE_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-inline-asm",
+    # LDS addresses are 32-bit integers turned into address-space-3 pointers; the host pass of
+    # hipcc, where pointers are 64 bits wide, warns about every such cast
+    "-Wno-int-to-pointer-cast",
     "-Rpass-analysis=kernel-resource-usage",
 ]
 RESOURCES_JSON = os.path.join(OBJ, "kernel_resources.json")
