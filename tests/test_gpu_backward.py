@@ -91,6 +91,30 @@ def test_random_metadata_backward(dtype, D, QB, KB, gpu_device):
             assert (t[:, :, seqlen:] == 0).all(), "rows beyond the sequence must get zero gradients"
 
 
+def test_sequences_of_length_zero_and_one(gpu_device):
+    """seqlen_orig = 0: nothing is attended, everything is zero (LSE -inf).  seqlen_orig = 1: row 0
+    attends key 0 alone, so O[0] = V[0], dV[0] = dO[0] and the softmax of one element has no
+    gradient with respect to its score."""
+    gen = torch.Generator().manual_seed(107)
+    B, H, S, D = 1, 2, 256, 64
+    q, k, v, dout = (torch.randn(B, H, S, D, generator=gen).to(torch.float16) for _ in range(4))
+    nb = torch.tensor([[[1, 2]]] * 1, dtype=torch.int32).expand(B, H, 2).contiguous()
+    idx = torch.tensor([[0, 0], [0, 1]], dtype=torch.int32).expand(B, H, 2, 2).contiguous()
+    tys = torch.tensor([[1, 0], [2, 1]], dtype=torch.int32).expand(B, H, 2, 2).contiguous()
+    dq, dk, dv, o, lse = run_fwd_bwd(q, k, v, dout, nb, idx, tys, 128, 128, 0, device=gpu_device)
+    for t in (dq, dk, dv, o):
+        assert (t == 0).all()
+    assert (lse == float("-inf")).all()
+    dq, dk, dv, o, lse = run_fwd_bwd(q, k, v, dout, nb, idx, tys, 128, 128, 1, device=gpu_device)
+    assert torch.equal(o[:, :, 0].cpu(), v[:, :, 0]) and (o[:, :, 1:] == 0).all()
+    assert torch.equal(dv[:, :, 0].cpu(), dout[:, :, 0]) and (dv[:, :, 1:] == 0).all()
+    # (dP and delta are the same sum in two summation orders: zero up to fp32 rounding)
+    assert dq.abs().max().item() <= 1e-3 and dk.abs().max().item() <= 1e-3
+    assert (dq[:, :, 1:] == 0).all() and (dk[:, :, 1:] == 0).all()
+    expect = (q[:, :, 0].float() * k[:, :, 0].float()).sum(-1) / 8.0
+    assert (lse[:, :, 0].cpu() - expect).abs().max().item() <= 1e-3 and (lse[:, :, 1:] == float("-inf")).all()
+
+
 def test_slab_counts_that_do_not_divide_over_the_xcds(gpu_device):
     """15 and 9 slabs: the kernels deal slabs to the 8 XCDs round-robin, so some XCDs get one slab
     more than others (forward and backward)."""
