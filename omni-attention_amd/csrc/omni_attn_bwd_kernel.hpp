@@ -327,32 +327,41 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
 
   // The steps of the walk in order, skipping what contributes nothing: MASKED slots, keys at or
   // beyond the sequence, CAUSAL steps entirely above the diagonal of this query block.
-  int gj = 0, gsub = 0;
+  // Inside a KV block the next step is the previous one moved on by STEP keys (both reasons to
+  // skip a step only get truer with the key index, so a block's steps are a prefix of it): that
+  // path is a handful of scalar instructions; the slots of the list are only read at the first
+  // step of a block.
+  int gj = 0;  // next slot of the list to look at
+  BwdStepInfo g_last = {0, kMasked, -1, 0, 0, false};
+  const int q_last = qb * QB + QB - 1;
   auto next_step = [&]() {
-    BwdStepInfo st = {0, kMasked, -1, 0, 0, false};
+    if (g_last.valid) {
+      const int r = g_last.row0 + STEP, sb = g_last.sub + 1;
+      const bool inside = bool(int(sb < SPB) & int(r < p.seqlen) & int(!(g_last.mode == kCausal && r > q_last)));
+      if (inside) {
+        g_last.row0 = r;
+        g_last.sub = sb;
+        return g_last;
+      }
+    }
+    g_last.valid = false;
     while (gj < nb) {
-      if (gsub == 0 && (gj & 63) == 0 && gj > 0) load_chunk(gj >> 6);
+      if ((gj & 63) == 0 && gj > 0) load_chunk(gj >> 6);
       const int ln = gj & 63;
       const int kvb = __builtin_amdgcn_readlane(mv_kvb, ln);
       const int mode = __builtin_amdgcn_readlane(mv_mode, ln);
       const int pid = __builtin_amdgcn_readlane(mv_pid, ln);
-      const int sub = gsub;
-      if (mode == kMasked || ++gsub == SPB) {
-        gsub = 0;
-        ++gj;
-      }
-      if (mode == kMasked) continue;
-      const int row0 = kvb * KB + sub * STEP;
-      if (row0 >= p.seqlen) continue;
-      if (mode == kCausal && row0 > qb * QB + QB - 1) continue;
-      st.row0 = row0;
-      st.mode = mode;
-      st.pid = pid;
-      st.sub = sub;
-      st.valid = true;
+      ++gj;
+      const int row0 = kvb * KB;
+      if (mode == kMasked || row0 >= p.seqlen || (mode == kCausal && row0 > q_last)) continue;
+      g_last.row0 = row0;
+      g_last.mode = mode;
+      g_last.pid = pid;
+      g_last.sub = 0;
+      g_last.valid = true;
       break;
     }
-    return st;
+    return g_last;
   };
   const uint32_t lds_tiles = lds_offset_of(lds16);
   auto issue_loads = [&](const BwdStepInfo& st, int set) {
@@ -614,53 +623,66 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
 
   // Pass 2: the matches in ascending (query block, slot) order, each as NSTEPS steps of STEP
   // query rows, skipping steps beyond the sequence and CAUSAL steps entirely above the diagonal.
-  int gw = -1, g_qb = 0, g_ch = -1, gsub = 0, g_mode = kMasked, g_pid = -1;  // word gw = (g_qb, g_ch)
+  // Inside a match the next step is the previous one moved on by STEP query rows (a CAUSAL step
+  // that is valid stays valid further down; only the end of the sequence can end a match early):
+  // that path is a handful of scalar instructions; the bitmap is only read at the first step of a
+  // match.
+  int gw = -1, g_qb = 0, g_ch = -1;  // word gw = (g_qb, g_ch)
   uint64_t gbits = 0;
   bool g_first = true;
+  BwdStepInfo g_last = {0, kMasked, -1, 0, 0, false};
   auto next_step = [&]() {
-    BwdStepInfo st = {0, kMasked, -1, 0, 0, false};
+    if (g_last.valid) {
+      const int r = g_last.row0 + STEP, sb = g_last.sub + 1;
+      if (bool(int(sb < NSTEPS) & int(r < p.seqlen))) {
+        g_last.row0 = r;
+        g_last.sub = sb;
+        return g_last;
+      }
+    }
+    g_last.valid = false;
     for (;;) {
-      if (gsub == 0) {
-        while (gbits == 0) {
-          if (++gw >= n_words) return st;
-          if (++g_ch == chunks) {
-            g_ch = 0;
-            ++g_qb;
-          }
-          const uint64_t m = sMatch[gw];
-          // (readfirstlane returns a signed int: go through uint32_t so that bit 31 does not sign-extend)
-          gbits = (uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(m >> 32))))) << 32) |
-                  uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(m)))));
-          g_first = true;
+      while (gbits == 0) {
+        if (++gw >= n_words) return g_last;
+        if (++g_ch == chunks) {
+          g_ch = 0;
+          ++g_qb;
         }
-        if (g_first) {
-          const int32_t info = __builtin_amdgcn_readfirstlane(sFirst[gw]);
-          g_mode = info & 3;
-          g_pid = g_mode == kPartial ? info >> 2 : -1;
-        } else {  // a further match in the same 64 slots
-          const size_t o = (meta_slab + g_qb) * p.max_blocks + g_ch * 64 + __builtin_ctzll(gbits);
-          const int32_t ty = load_uniform(p.types + o);
-          g_pid = has_partial ? load_uniform(p.partial_idx + o) : -1;
-          g_mode = bwd_slot_mode(ty, g_pid, has_partial, p.num_partial);
-        }
+        const uint64_t m = sMatch[gw];
+        // (readfirstlane returns a signed int: go through uint32_t so that bit 31 does not sign-extend)
+        gbits = (uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(m >> 32))))) << 32) |
+                uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(m)))));
+        g_first = true;
       }
-      const int qb = g_qb;
-      const int sub = gsub;
-      if (++gsub == NSTEPS) {
-        gsub = 0;
-        gbits &= gbits - 1;
-        g_first = false;
+      int mode, pid;
+      if (g_first) {
+        const int32_t info = __builtin_amdgcn_readfirstlane(sFirst[gw]);
+        mode = info & 3;
+        pid = mode == kPartial ? info >> 2 : -1;
+      } else {  // a further match in the same 64 slots
+        const size_t o = (meta_slab + g_qb) * p.max_blocks + g_ch * 64 + __builtin_ctzll(gbits);
+        const int32_t ty = load_uniform(p.types + o);
+        pid = has_partial ? load_uniform(p.partial_idx + o) : -1;
+        mode = bwd_slot_mode(ty, pid, has_partial, p.num_partial);
       }
-      const int q0 = qb * QB + sub * STEP;
-      if (q0 >= p.seqlen) continue;
-      if (g_mode == kCausal && q0 + STEP - 1 < kvb * KB) continue;
-      st.row0 = q0;
-      st.mode = g_mode;
-      st.pid = g_pid;
-      st.blk = qb;
-      st.sub = sub;
-      st.valid = true;
-      return st;
+      gbits &= gbits - 1;
+      g_first = false;
+      // first step of the match that contributes: CAUSAL steps entirely above the diagonal and
+      // steps beyond the sequence do not
+      int sub = 0;
+      if (mode == kCausal) {
+        const int below = kvb * KB - (g_qb * QB + STEP - 1);  // rows of the block before the first useful step
+        sub = below > 0 ? (below + STEP - 1) / STEP : 0;
+      }
+      const int q0 = g_qb * QB + sub * STEP;
+      if (sub >= NSTEPS || q0 >= p.seqlen) continue;
+      g_last.row0 = q0;
+      g_last.mode = mode;
+      g_last.pid = pid;
+      g_last.blk = g_qb;
+      g_last.sub = sub;
+      g_last.valid = true;
+      return g_last;
     }
   };
   const uint32_t lds_tiles = lds_offset_of(lds16);
