@@ -291,6 +291,84 @@ def fixed_cost_study(dev, seed, steps, warmup):
             "rows": rows}
 
 
+def power_study(dev, seed, steps, warmup):
+    """What the clock does to the figures.  (1) The library's matrix-instruction loop with eight
+    operand sets, alone and with the forward kernel's LDS operand reads and softmax vector work
+    beside it: rate and the shader clock one of its waves saw.  (2) The forward kernel on
+    c2_interleaved with its real operands, with V zero and with all operands zero: the same
+    instructions in the same order, but matrix cores and data paths that toggle fewer bits draw less
+    power and the device grants a higher clock."""
+    import torch
+
+    import omni_attn_capi
+    from baseline_configs import make_workload
+
+    stream = torch.cuda.current_stream(dev)
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    ticks = torch.zeros(2, dtype=torch.int64, device=dev)
+    names = {0: "mfma only, eight operand sets in turn", 1: "mfma + A operand from LDS",
+             2: "mfma + softmax vector work", 3: "mfma + A operand from LDS + softmax vector work"}
+    mixes = []
+    for mix in range(4):
+        iters = 20000
+        t_end = time.perf_counter() + 0.25
+        while time.perf_counter() < t_end:
+            for _ in range(3):
+                omni_attn_capi.mfma_mix_probe(mix, iters, sink, None, stream.cuda_stream)
+            torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            flops = omni_attn_capi.mfma_mix_probe(mix, iters, sink, ticks, stream.cuda_stream)
+            b.record(stream)
+            torch.cuda.synchronize()
+            tf = flops / (a.elapsed_time(b) * 1e-3) / 1e12
+            cyc, rt = (int(x) for x in ticks.tolist())
+            if best is None or tf > best["tflops"]:
+                best = {"mix": names[mix], "tflops": tf, "shader_clock_mhz": 100.0 * cyc / max(rt, 1),
+                        "frac_of_rated_peak": tf / MFMA_PEAK_TFLOPS}
+        best["mfma_busy_at_that_clock"] = best["tflops"] / (MFMA_PEAK_TFLOPS * best["shader_clock_mhz"] / 2400.0)
+        mixes.append(best)
+
+    w = make_workload("c2_interleaved", seed=seed)
+    m = w.block_mask
+    B, H, S, D = w.q.shape
+    nb, idx, tys = (t.to(dev) for t in (m.kv_num_blocks, m.kv_indices, m.block_mask_types))
+    o = torch.empty(w.q.shape, dtype=w.dtype, device=dev)
+    lse = torch.empty(B, H, S, dtype=torch.float32, device=dev)
+    rows = []
+    for what in ("operands as in the benchmark (standard normal)", "V zero", "Q, K and V zero"):
+        q, k, v = (t.to(dev) for t in (w.q, w.k, w.v))
+        if what != "operands as in the benchmark (standard normal)":
+            v = torch.zeros_like(v)
+        if what == "Q, K and V zero":
+            q, k = torch.zeros_like(q), torch.zeros_like(k)
+
+        def step():
+            omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, None, None,
+                               stream=stream.cuda_stream)
+
+        t_end = time.perf_counter() + 0.25
+        while time.perf_counter() < t_end:
+            for _ in range(10):
+                step()
+            torch.cuda.synchronize()
+        st = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        en = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        for i in range(steps):
+            st[i].record(stream)
+            step()
+            en[i].record(stream)
+        torch.cuda.synchronize()
+        ms = statistics.median(a.elapsed_time(b) for a, b in zip(st, en))
+        tf = w.effective_flops / (ms * 1e-3) / 1e12
+        rows.append({"operands": what, "kernel_us": ms * 1e3, "tflops": tf, "frac_of_rated_peak": tf / MFMA_PEAK_TFLOPS})
+    return {"study": "clock under load: instruction mixes of the probe loop, and the forward kernel on "
+                     "c2_interleaved (B=2 H=32 S=4096 D=128 bf16) with operands that toggle fewer bits",
+            "probe_mixes": mixes, "forward_c2_interleaved": rows}
+
+
 def extra_workload(name, seed, dev, steps, warmup, backward=False):
     """Kernel time of another workload, or of the backward of a workload (HIP events on the launch
     stream, clock already settled)."""
@@ -372,6 +450,10 @@ def main(argv=None):
     ap.add_argument("--fixed-cost", action="store_true",
                     help="instead of the workload: c2_interleaved with its lists repeated, its types all "
                          "FULL, its blocks spread evenly (fixed cost / mask cost / imbalance of a launch)")
+    ap.add_argument("--power-study", action="store_true",
+                    help="instead of the workload: the probe loop with the forward kernel's LDS reads and "
+                         "vector work beside the matrix instructions (rate and shader clock), and the forward "
+                         "kernel with zero operands")
     ap.add_argument("--sweep-bands", action="store_true",
                     help="instead of the workload: kernel time against the number of listed blocks")
     args = ap.parse_args(argv)
@@ -396,6 +478,9 @@ def main(argv=None):
     omni_attn_capi.load_library()  # fail loudly when the HIP library is missing
     if args.sweep_bands:
         print(json.dumps(band_sweep(dev, min(args.steps, 30), min(args.warmup, 5))))
+        return 0
+    if args.power_study:
+        print(json.dumps(power_study(dev, args.seed, min(args.steps, 60), min(args.warmup, 10))))
         return 0
     if args.fixed_cost:
         print(json.dumps(fixed_cost_study(dev, args.seed, min(args.steps, 60), min(args.warmup, 10))))

@@ -231,6 +231,20 @@ int omni_attn_bwd_noalloc_gfx950(const void* q, const void* k, const void* v, co
 int omni_attn_mfma_peak_probe_gfx950(int dtype, int iters, float* sink, double* flops_out,
                                      void* stream);
 
+/*
+ * Measurement aid (no counterpart in the reference): the same bf16 loop with eight operand sets
+ * in turn and, by the bits of `mix`, the forward kernel's other work beside the matrix
+ * instructions: 1 = the A operand of every instruction is read from LDS (1 KiB per wave and
+ * instruction), 2 = the vector work of a softmax (per instruction one fma, exp2 and add, per two
+ * a max3 and a 16-bit pack).  No barriers, tile loads or bookkeeping: rate and clock of such a
+ * loop show what each kind of work costs beside the matrix instructions.
+ * `ticks` (device memory, two 64-bit words, may be NULL) receives from one wave the shader
+ * cycles and the 100 MHz real-time ticks its loop took: their ratio x 100 is the shader clock
+ * in MHz under this load.  Allocates nothing.
+ */
+int omni_attn_mfma_mix_probe_gfx950(int mix, int iters, float* sink, unsigned long long* ticks,
+                                    double* flops_out, void* stream);
+
 /* Static description of a return code (never NULL). */
 const char* omni_attn_status_string(int status);
 

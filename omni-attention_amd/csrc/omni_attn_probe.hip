@@ -73,6 +73,85 @@ __global__ void __launch_bounds__(kThreads, 2) mfma_peak_kernel(int iters, float
   if (s == 12345.678f) sink[0] = s;  // keeps the accumulators alive; practically never true
 }
 
+
+// ---- the same loop with the forward kernel's other work beside the matrix instructions -----
+//
+// The device lowers its clock until the power fits, and how far depends on everything the loop
+// does, operand values included.  This variant rotates eight operand sets, can take the A
+// operand of every MFMA from LDS (16 bytes per lane: 1 KiB per wave and MFMA, the forward
+// kernel's rate, fetched one round ahead) and can run the vector work of a softmax beside it
+// (per MFMA one fma, one exp2 and one add on a value an earlier MFMA produced; per two MFMAs a
+// max3 and a 16-bit pack), scheduled by the compiler.  No barriers, tile loads or bookkeeping:
+// rate and clock of such a loop show what each kind of work costs beside the matrix
+// instructions.  One wave also reports the shader clock it saw: s_memtime ticks (shader cycles)
+// per s_memrealtime tick (100 MHz).
+constexpr int kMixLds = 1;
+constexpr int kMixSoftmax = 2;
+constexpr int kMixSets = 8;
+
+template <int MIX>
+__global__ void __launch_bounds__(kThreads, 2) mfma_mix_kernel(int iters, float* sink, unsigned long long* ticks) {
+  __shared__ u32x4_t tile[2048];  // 32 KiB: 8 KiB per wave, 8 fragments of 1 KiB
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  for (uint32_t i = tid; i < 2048u; i += kThreads)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) tile[i][j] = operand_word(i + 2048u * blockIdx.x, uint32_t(j), true);
+  __syncthreads();
+  u32x4_t a[kMixSets], b[kMixSets];
+#pragma unroll
+  for (int i = 0; i < kMixSets; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      a[i][j] = operand_word(lane, uint32_t(8 * i + j), true);
+      b[i][j] = operand_word(lane + 977u * blockIdx.x, uint32_t(8 * i + 4 + j), true);
+    }
+  f32x16_t acc[kMixSets];
+#pragma unroll
+  for (int c = 0; c < kMixSets; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[c][r] = 0.f;
+  const u32x4_t* frag = tile + wave * 512u + lane;
+  float sum = 0.f, mx = -INFINITY, e_prev = 0.f, t_prev = 0.f;
+  uint32_t packed = 0u;
+  const unsigned long long t0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+  for (int it = 0; it < iters; ++it) {
+    if constexpr ((MIX & kMixLds) != 0) {
+      // the fragments the next round multiplies; the asm statement keeps the reads in the loop
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int c = 0; c < kMixSets; ++c) a[c] = frag[((it + c) & 7) * 64];
+    }
+#pragma unroll
+    for (int c = 0; c < kMixSets; ++c) {
+      acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[c]),
+                                                       __builtin_bit_cast(bf16x8_t, b[c]), acc[c], 0, 0, 0);
+      if constexpr ((MIX & kMixSoftmax) != 0) {
+        const float t = __builtin_fmaf(acc[(c + 4) % kMixSets][c], 9.765625e-4f, -0.25f);
+        const float e = __builtin_amdgcn_exp2f(t);
+        sum += e;
+        if (c & 1) {
+          mx = __builtin_fmaxf(__builtin_fmaxf(mx, t), t_prev);
+          asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(packed) : "v"(e), "v"(e_prev));
+        }
+        e_prev = e;
+        t_prev = t;
+        asm volatile("" : "+v"(sum), "+v"(mx));
+      }
+    }
+  }
+  const unsigned long long t1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+  float s = sum + mx + __builtin_bit_cast(float, packed);
+#pragma unroll
+  for (int c = 0; c < kMixSets; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += acc[c][r];
+  if (s == 12345.678f) sink[0] = s;
+  if (tid == 0 && blockIdx.x == gridDim.x / 2 && ticks != nullptr) {
+    ticks[0] = t1 - t0;
+    ticks[1] = r1 - r0;
+  }
+}
+
 }  // namespace
 
 extern "C" int omni_attn_mfma_peak_probe_gfx950(int dtype, int iters, float* sink, double* flops_out,
@@ -92,5 +171,24 @@ extern "C" int omni_attn_mfma_peak_probe_gfx950(int dtype, int iters, float* sin
     return OMNI_ATTN_ERR_LAUNCH;
   // waves x iterations x chains x (2 * 32 * 32 * 16) flop
   *flops_out = double(grid) * (kThreads / 64) * double(iters) * kChains * 32768.0;
+  return OMNI_ATTN_OK;
+}
+
+
+extern "C" int omni_attn_mfma_mix_probe_gfx950(int mix, int iters, float* sink, unsigned long long* ticks,
+                                               double* flops_out, void* stream) {
+  if (!sink || !flops_out) return OMNI_ATTN_ERR_NULL_POINTER;
+  if (mix < 0 || mix > 3 || iters <= 0 || iters > (1 << 24)) return OMNI_ATTN_ERR_BAD_SHAPE;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    return OMNI_ATTN_ERR_LAUNCH;
+  const unsigned grid = unsigned(cus) * kWorkgroupsPerCu;
+  const void* kerns[4] = {reinterpret_cast<const void*>(mfma_mix_kernel<0>), reinterpret_cast<const void*>(mfma_mix_kernel<1>),
+                          reinterpret_cast<const void*>(mfma_mix_kernel<2>), reinterpret_cast<const void*>(mfma_mix_kernel<3>)};
+  void* args[] = {&iters, &sink, &ticks};
+  if (hipLaunchKernel(kerns[mix], dim3(grid), dim3(kThreads), args, 0, static_cast<hipStream_t>(stream)) != hipSuccess)
+    return OMNI_ATTN_ERR_LAUNCH;
+  *flops_out = double(grid) * (kThreads / 64) * double(iters) * kMixSets * 32768.0;
   return OMNI_ATTN_OK;
 }

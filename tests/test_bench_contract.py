@@ -65,3 +65,25 @@ def test_json_line_has_the_contract_fields(gpu_device):
     assert 500.0 < rf["measured_mfma_peak"] < 2600.0 and "measured_at_head" in rf["traffic_provenance"]
     cb = d["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]
+
+
+@pytest.mark.gpu
+def test_mix_probe_reports_a_rate_and_a_plausible_clock(gpu_device):
+    import torch
+
+    import omni_attn_capi
+
+    sink = torch.zeros(1, dtype=torch.float32, device=gpu_device)
+    ticks = torch.zeros(2, dtype=torch.int64, device=gpu_device)
+    for mix in range(4):
+        ticks.zero_()
+        flops = omni_attn_capi.mfma_mix_probe(mix, 2000, sink, ticks)
+        torch.cuda.synchronize()
+        cycles, real = (int(x) for x in ticks.tolist())
+        assert flops == 512 * 4 * 2000 * 8 * 32768.0 * (torch.cuda.get_device_properties(gpu_device).multi_processor_count / 256)
+        assert cycles >= 2000 * 8 * 16 and real > 0       # 8 matrix instructions of 32 cycles, two waves per SIMD
+        assert 500.0 < 100.0 * cycles / real < 3000.0    # shader clock in MHz
+    with pytest.raises(RuntimeError):
+        omni_attn_capi.mfma_mix_probe(4, 10, sink, None)
+    with pytest.raises(RuntimeError):
+        omni_attn_capi.mfma_mix_probe(0, 10, sink, torch.zeros(2, dtype=torch.int32, device=gpu_device))
