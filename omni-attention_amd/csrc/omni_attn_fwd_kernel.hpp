@@ -155,10 +155,11 @@ __device__ __forceinline__ float pair_sum(float x) {
 template <bool BF16, int D, int QB, int KB>
 struct FwdTraits {
   static constexpr int kThreads = QB * 2;  // QB/32 waves of 64 lanes
-  // Keys per step.  A 64-row query block has half the waves and would leave LDS room for
-  // only two workgroups per CU (one wave per SIMD) with 64-key tiles: it steps by 32 keys,
-  // four workgroups fit and every SIMD has two waves again.
-  static constexpr int kStep = QB == 64 ? 32 : 64;
+  // Keys per step.  A 64-row query block has half the waves; at D = 128 its 64-key tiles would
+  // leave LDS room for only two workgroups per CU (one wave per SIMD): it steps by 32 keys, four
+  // workgroups fit and every SIMD has two waves again.  At D <= 64 four workgroups fit with 64-key
+  // tiles, and a step has twice the matrix work per barrier.
+  static constexpr int kStep = (QB == 64 && D == 128) ? 32 : 64;
   static constexpr int kTileElems = kStep * D;
   // K tiles, V tiles, one mask word per row and 32 keys, one mask byte per row and key in transit
   static constexpr size_t kLdsBytes = size_t(2) * 2 * kTileElems * sizeof(uint16_t) +
