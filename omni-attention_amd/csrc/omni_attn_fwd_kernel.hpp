@@ -141,10 +141,23 @@ __device__ __forceinline__ void pair_split(float x, float& lo, float& hi) {
   lo = __builtin_bit_cast(float, r0);
   hi = __builtin_bit_cast(float, r1);
 }
+// Maximum of values that are never NaN, as exactly one v_max_f32 / v_max3_f32 (the library
+// function also quiets signalling NaNs: one more instruction for every operand the compiler
+// knows nothing about).
+__device__ __forceinline__ float vmax(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float vmax3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
 __device__ __forceinline__ float pair_max(float x) {
   float lo, hi;
   pair_split(x, lo, hi);
-  return fmaxf(lo, hi);
+  return vmax(lo, hi);
 }
 __device__ __forceinline__ float pair_sum(float x) {
   float lo, hi;
@@ -459,9 +472,10 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
 
   // Does this wave's 32 x STEP tile of the step need no mask at all?  (wave-uniform)
   auto unmasked = [&](const StepInfo& si) {
-    if (si.row0 + STEP > p.seqlen) return false;
-    if (si.mode == kFull) return true;
-    return si.mode == kCausal && si.row0 + STEP - 1 <= q_wave_min;
+    const bool inside = si.row0 + STEP <= p.seqlen;  // (written without branches: scalar selects)
+    const bool full = si.mode == kFull;
+    const bool below = (si.mode == kCausal) & (si.row0 + STEP - 1 <= q_wave_min);
+    return inside & (full | below);
   };
 
   // LDS operand fetches.  K: rows 32t + c of the tile at k-step s.
@@ -572,7 +586,25 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     });
   };
 
-  auto body = [&](auto set_c, auto first_c, int k_row0, int v_row0) {
+  // The first operands of an iteration are fetched right after the barrier, ahead of everything
+  // else that happens between two bodies: their LDS latency runs under that bookkeeping.
+  auto body_prefetch = [&](auto set_c, auto first_c, u32x4_t* opq) {
+    constexpr int SET = decltype(set_c)::value;
+    constexpr int NPV = decltype(first_c)::value != 0 ? 0 : NPV_ALL;
+    constexpr int NS = NQK + NPV;
+    constexpr int PF = PF_ALL < NS ? PF_ALL : NS;
+    const uint16_t* tK = sK + (SET ^ 1) * TILE;
+    const uint16_t* tV = sV + (SET ^ 1) * TILE;
+    static_for<PF>([&](auto nc) {
+      constexpr int n = decltype(nc)::value;
+      if constexpr (n < NPV) {
+        opq[n] = v_frag(tV, n);
+      } else {
+        opq[n] = k_frag(tK, (n - NPV) / NTL, (n - NPV) % NTL);
+      }
+    });
+  };
+  auto body = [&](auto set_c, auto first_c, int k_row0, int v_row0, u32x4_t* opq) {
     constexpr int SET = decltype(set_c)::value;
     // The first iteration of a walk has no previous step: no PV slots.
     constexpr int NPV = decltype(first_c)::value != 0 ? 0 : NPV_ALL;
@@ -587,24 +619,23 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     const uint16_t* tV = sV + (SET ^ 1) * TILE;
     auto operand = [&](int n) { return n < NPV ? v_frag(tV, n) : k_frag(tK, (n - NPV) / NTL, (n - NPV) % NTL); };
 
-    u32x4_t opq[PF];
-#pragma unroll
-    for (int n = 0; n < PF; ++n) opq[n] = operand(n);
-
-    float mxa = -INFINITY, mxb = -INFINITY, m_ref = 0.f, rs0 = 0.f, rs1 = 0.f;
+    float mxa, mxb, m_ref = 0.f, rs0, rs1;
     auto vector_chunk = [&](auto uc) {
       constexpr int u = decltype(uc)::value;
       if constexpr (u < 0) {
       } else if constexpr (u < NMX) {
-        static_for<8>([&](auto ec) {
-          constexpr int e = 8 * u + decltype(ec)::value;
-          if constexpr ((u & 1) != 0) {
-            mxb = fmaxf(mxb, st[SET][e / 16][e % 16]);
+        static_for<4>([&](auto ec) {
+          constexpr int e = 8 * u + 2 * decltype(ec)::value;
+          if constexpr (u == 0 && e == 0) {
+            mxa = vmax(st[SET][0][0], st[SET][0][1]);
+          } else if constexpr (u == 1 && e == 8) {
+            mxb = vmax(st[SET][0][8], st[SET][0][9]);
+          } else if constexpr ((u & 1) != 0) {
+            mxb = vmax3(mxb, st[SET][e / 16][e % 16], st[SET][e / 16][e % 16 + 1]);
           } else {
-            mxa = fmaxf(mxa, st[SET][e / 16][e % 16]);
+            mxa = vmax3(mxa, st[SET][e / 16][e % 16], st[SET][e / 16][e % 16 + 1]);
           }
         });
-        pin(mxa, mxb);
       } else if constexpr (u == NMX) {
         // The reference point m_run of the exponentials only has to stay within 2^kSlack of
         // the true running max (P then stays below 2^kSlack, exact in fp32 and well inside
@@ -613,11 +644,11 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
         // result is the same sum with a different common factor.  (Written without
         // branches: an unmoved reference gives a factor of exactly 1, or of 0 for a row that
         // has not seen a key yet and whose sums are still 0.)
-        const float mx = pair_max(fmaxf(mxa, mxb));  // the row lives in lanes c and c+32
+        const float mx = pair_max(vmax(mxa, mxb));  // the row lives in lanes c and c+32
         const float m_cand = mx * p.sl2;
         const uint64_t movers = __builtin_amdgcn_ballot_w64(m_cand > m_run + kSlack);
         const bool move = movers != 0;
-        const float m_new = move ? fmaxf(m_run, m_cand) : m_run;
+        const float m_new = move ? vmax(m_run, m_cand) : m_run;
         m_ref = m_new == -INFINITY ? 0.f : m_new;
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
         l_run *= alpha;
@@ -630,8 +661,13 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
         constexpr int t = i / 8, r = 2 * (i % 8);
         const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[SET][t][r], p.sl2, -m_ref));
         const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[SET][t][r + 1], p.sl2, -m_ref));
-        rs0 += p0;
-        rs1 += p1;
+        if constexpr (i == 0) {
+          rs0 = p0;
+          rs1 = p1;
+        } else {
+          rs0 += p0;
+          rs1 += p1;
+        }
         uint32_t packed = pack2<BF16>(p0, p1);
         pin(packed);
         pb[SET][t][r >> 3][(r & 7) >> 1] = packed;
@@ -696,24 +732,31 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     constexpr int SET = decltype(set_c)::value;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's tile loads have landed
     __syncthreads();
-    if (rescale_pending != 0) {
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) ot[dt][r] *= alpha_pending;
-      rescale_pending = 0;
-    }
-    if (p.softcap > 0.f) apply_softcap(IntC<SET>{});
-    if (!unmasked(cur)) apply_mask(IntC<SET>{}, cur);
+    u32x4_t opq[PF_ALL];
+    body_prefetch(IntC<SET>{}, first_c, opq);
+    // The common step -- every score allowed, no rescale owed, no PARTIAL tile ahead, no soft cap
+    // -- goes from the barrier into the slots over one scalar condition and one branch.
     const bool next_partial = it + 1 < nsteps && nxt.mode == kPartial;
-    if (next_partial) {
-      if (packed_tiles) {
-        prefetch_mask_words(it + 1, nxt);
-      } else {
-        prefetch_mask_bytes(it + 1, nxt);
+    const bool plain = (rescale_pending == 0) & !(p.softcap > 0.f) & unmasked(cur) & !next_partial;
+    if (!plain) {
+      if (rescale_pending != 0) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) ot[dt][r] *= alpha_pending;
+        rescale_pending = 0;
+      }
+      if (p.softcap > 0.f) apply_softcap(IntC<SET>{});
+      if (!unmasked(cur)) apply_mask(IntC<SET>{}, cur);
+      if (next_partial) {
+        if (packed_tiles) {
+          prefetch_mask_words(it + 1, nxt);
+        } else {
+          prefetch_mask_bytes(it + 1, nxt);
+        }
       }
     }
-    body(IntC<SET>{}, first_c, nn.row0, cur.row0);
+    body(IntC<SET>{}, first_c, nn.row0, cur.row0, opq);
     if (next_partial && !packed_tiles) stage_mask_bits();
     const StepInfo n3 = step_info(it + 3);
     cur = nxt;
