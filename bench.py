@@ -369,6 +369,35 @@ def power_study(dev, seed, steps, warmup):
             "probe_mixes": mixes, "forward_c2_interleaved": rows}
 
 
+def issue_study(dev):
+    """How much softmax vector work fits under a matrix instruction on one SIMD: the issue probe
+    (one workgroup on one compute unit; groups of one bf16 32x32x16 MFMA + n v_fma_f32 + e v_exp_f32
+    on registers of their own) at one and two waves per SIMD.  Cycles per group and SIMD; a matrix
+    instruction alone takes 32."""
+    import torch
+
+    import omni_attn_capi
+
+    ticks = torch.zeros(17, dtype=torch.int64, device=dev)
+    iters = 2048
+    rows = []
+    for n_exp in (0, 1, 2):
+        for n_plain in (0, 2, 4, 6, 8):
+            row = {"v_fma_f32_per_mfma": n_plain, "v_exp_f32_per_mfma": n_exp}
+            for waves in (1, 2):
+                best = None
+                for _ in range(3):
+                    omni_attn_capi.issue_probe(n_plain, n_exp, waves, iters, ticks)
+                    torch.cuda.synchronize()
+                    t = ticks.tolist()
+                    span = max(t[2 * w + 1] for w in range(4 * waves)) - min(t[2 * w] for w in range(4 * waves))
+                    cyc = span / (4.0 * iters * waves)
+                    best = cyc if best is None else min(best, cyc)
+                row["cycles_per_group_per_simd_%dw" % waves] = best
+            rows.append(row)
+    return {"study": "vector work beside the matrix instructions of one SIMD (issue probe)", "rows": rows}
+
+
 def extra_workload(name, seed, dev, steps, warmup, backward=False):
     """Kernel time of another workload, or of the backward of a workload (HIP events on the launch
     stream, clock already settled)."""
@@ -454,6 +483,9 @@ def main(argv=None):
                     help="instead of the workload: the probe loop with the forward kernel's LDS reads and "
                          "vector work beside the matrix instructions (rate and shader clock), and the forward "
                          "kernel with zero operands")
+    ap.add_argument("--issue-study", action="store_true",
+                    help="instead of the workload: cycles per matrix instruction and SIMD with 0..8 plain and "
+                         "0..2 transcendental vector instructions issued beside each (one compute unit)")
     ap.add_argument("--sweep-bands", action="store_true",
                     help="instead of the workload: kernel time against the number of listed blocks")
     args = ap.parse_args(argv)
@@ -478,6 +510,9 @@ def main(argv=None):
     omni_attn_capi.load_library()  # fail loudly when the HIP library is missing
     if args.sweep_bands:
         print(json.dumps(band_sweep(dev, min(args.steps, 30), min(args.warmup, 5))))
+        return 0
+    if args.issue_study:
+        print(json.dumps(issue_study(dev)))
         return 0
     if args.power_study:
         print(json.dumps(power_study(dev, args.seed, min(args.steps, 60), min(args.warmup, 10))))

@@ -245,6 +245,19 @@ int omni_attn_mfma_peak_probe_gfx950(int dtype, int iters, float* sink, double* 
 int omni_attn_mfma_mix_probe_gfx950(int mix, int iters, float* sink, unsigned long long* ticks,
                                     double* flops_out, void* stream);
 
+/*
+ * Measurement aid (no counterpart in the reference): one workgroup on one compute unit,
+ * `waves_per_simd` (1 or 2) waves on every SIMD, each running `iters` x 4 groups of one bf16
+ * 32x32x16 matrix instruction followed by `n_plain` (0, 2, 4, 6 or 8) v_fma_f32 and `n_exp`
+ * (0, 1 or 2) v_exp_f32 on registers of their own.  `ticks` (device memory, at least 17 64-bit
+ * words) receives for wave w the shader cycle counter at the start (word 2w) and the end (word
+ * 2w + 1) of its loop: (latest end - earliest start) / (4 * iters * waves_per_simd) is the time
+ * one SIMD needs per group -- how much vector work fits under a matrix instruction.
+ * Allocates nothing.
+ */
+int omni_attn_issue_probe_gfx950(int n_plain, int n_exp, int waves_per_simd, int iters,
+                                 unsigned long long* ticks, void* stream);
+
 /* Static description of a return code (never NULL). */
 const char* omni_attn_status_string(int status);
 

@@ -152,6 +152,70 @@ __global__ void __launch_bounds__(kThreads, 2) mfma_mix_kernel(int iters, float*
   }
 }
 
+// ---- what the vector pipe can do beside the matrix instructions of one SIMD --------------------
+//
+// One workgroup on one compute unit, 1 or 2 waves per SIMD.  Every wave runs a loop of groups:
+// one MFMA (four accumulators in turn, so no instruction waits for another), then NP plain
+// vector instructions (v_fma_f32) and NE transcendental ones (v_exp_f32) on registers the
+// matrix instructions do not touch.  Cycles per group and SIMD, over NP and NE, show how much
+// softmax work fits under a matrix instruction before the vector pipe becomes the longer one.
+template <int NP, int NE>
+__global__ void __launch_bounds__(512) issue_probe_kernel(int iters, unsigned long long* ticks, float seed) {
+  f32x16_t acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[i][j] = seed * float(j);
+  u32x4_t a, b;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    a[j] = operand_word(threadIdx.x, uint32_t(j), true);
+    b[j] = operand_word(threadIdx.x + 977u, uint32_t(4 + j), true);
+  }
+  float v[8], e[2];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = seed + float(threadIdx.x) * 1e-3f + float(j);
+  e[0] = seed;
+  e[1] = -seed;
+  __syncthreads();
+  const unsigned long long t0 = __builtin_amdgcn_s_memtime();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                       __builtin_bit_cast(bf16x8_t, b), acc[m], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < NP; ++j) asm volatile("v_fma_f32 %0, %0, %0, %0" : "+v"(v[j]));
+#pragma unroll
+      for (int j = 0; j < NE; ++j) asm volatile("v_exp_f32 %0, %0" : "+v"(e[j]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  const unsigned long long t1 = __builtin_amdgcn_s_memtime();
+  if ((threadIdx.x & 63u) == 0u) {
+    ticks[2 * (threadIdx.x >> 6)] = t0;
+    ticks[2 * (threadIdx.x >> 6) + 1] = t1;
+  }
+  float s = e[0] + e[1];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) s += acc[i][j];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) s += v[j];
+  if (s == 12345.678f) ticks[16] = 1;  // keeps the results alive; practically never true
+}
+
+template <int NP>
+const void* issue_probe_for(int n_exp) {
+  switch (n_exp) {
+    case 0: return reinterpret_cast<const void*>(issue_probe_kernel<NP, 0>);
+    case 1: return reinterpret_cast<const void*>(issue_probe_kernel<NP, 1>);
+    case 2: return reinterpret_cast<const void*>(issue_probe_kernel<NP, 2>);
+    default: return nullptr;
+  }
+}
+
 }  // namespace
 
 extern "C" int omni_attn_mfma_peak_probe_gfx950(int dtype, int iters, float* sink, double* flops_out,
@@ -190,5 +254,28 @@ extern "C" int omni_attn_mfma_mix_probe_gfx950(int mix, int iters, float* sink, 
   if (hipLaunchKernel(kerns[mix], dim3(grid), dim3(kThreads), args, 0, static_cast<hipStream_t>(stream)) != hipSuccess)
     return OMNI_ATTN_ERR_LAUNCH;
   *flops_out = double(grid) * (kThreads / 64) * double(iters) * kMixSets * 32768.0;
+  return OMNI_ATTN_OK;
+}
+
+
+extern "C" int omni_attn_issue_probe_gfx950(int n_plain, int n_exp, int waves_per_simd, int iters,
+                                            unsigned long long* ticks, void* stream) {
+  if (!ticks) return OMNI_ATTN_ERR_NULL_POINTER;
+  if (n_plain < 0 || n_plain > 8 || (n_plain & 1) || n_exp < 0 || n_exp > 2 || waves_per_simd < 1 ||
+      waves_per_simd > 2 || iters <= 0 || iters > (1 << 20))
+    return OMNI_ATTN_ERR_BAD_SHAPE;
+  const void* kern = nullptr;
+  switch (n_plain) {
+    case 0: kern = issue_probe_for<0>(n_exp); break;
+    case 2: kern = issue_probe_for<2>(n_exp); break;
+    case 4: kern = issue_probe_for<4>(n_exp); break;
+    case 6: kern = issue_probe_for<6>(n_exp); break;
+    default: kern = issue_probe_for<8>(n_exp); break;
+  }
+  float seed = 1e-3f;
+  void* args[] = {&iters, &ticks, &seed};
+  if (hipLaunchKernel(kern, dim3(1), dim3(256u * unsigned(waves_per_simd)), args, 0,
+                      static_cast<hipStream_t>(stream)) != hipSuccess)
+    return OMNI_ATTN_ERR_LAUNCH;
   return OMNI_ATTN_OK;
 }

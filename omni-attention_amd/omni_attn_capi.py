@@ -28,6 +28,7 @@ EXPORTED_SYMBOLS = (
     "omni_attn_bwd_noalloc_max_rows",
     "omni_attn_mfma_peak_probe_gfx950",
     "omni_attn_mfma_mix_probe_gfx950",
+    "omni_attn_issue_probe_gfx950",
     "omni_attn_status_string",
     "omni_attn_last_hip_error",
     "omni_attn_abi_version",
@@ -63,6 +64,8 @@ def load_library() -> ctypes.CDLL:
         lib.omni_attn_status_string.restype = ctypes.c_char_p
         lib.omni_attn_status_string.argtypes = [i32]
         lib.omni_attn_last_hip_error.restype = i32
+        lib.omni_attn_issue_probe_gfx950.restype = i32
+        lib.omni_attn_issue_probe_gfx950.argtypes = [i32, i32, i32, i32, vp, vp]
         lib.omni_attn_abi_version.restype = i32
         _lib = lib
     return _lib
@@ -101,6 +104,22 @@ def mfma_mix_probe(mix: int, iters: int, sink: torch.Tensor, ticks: Optional[tor
     if rc != 0:
         raise RuntimeError("omni_attn_mfma_mix_probe_gfx950: %s (status %d)" % (status_string(rc), rc))
     return flops.value
+
+
+def issue_probe(n_plain: int, n_exp: int, waves_per_simd: int, iters: int, ticks: torch.Tensor,
+                stream: Optional[int] = None) -> None:
+    """Enqueue the issue probe: one workgroup, `waves_per_simd` waves per SIMD, groups of one matrix
+    instruction + `n_plain` v_fma_f32 + `n_exp` v_exp_f32.  `ticks`: at least 17 int64 on the GPU;
+    wave w's loop started at ticks[2w] and ended at ticks[2w + 1] (shader cycles)."""
+    if not (ticks.is_cuda and ticks.dtype == torch.int64 and ticks.numel() >= 17 and ticks.is_contiguous()):
+        raise RuntimeError("ticks must be a contiguous int64 GPU tensor with at least 17 elements")
+    if stream is None:
+        stream = torch.cuda.current_stream(ticks.device).cuda_stream
+    with torch.cuda.device(ticks.device):
+        rc = load_library().omni_attn_issue_probe_gfx950(n_plain, n_exp, waves_per_simd, iters, ticks.data_ptr(),
+                                                         stream)
+    if rc != 0:
+        raise RuntimeError("omni_attn_issue_probe_gfx950: %s (status %d)" % (status_string(rc), rc))
 
 
 def _ptr(t: Optional[torch.Tensor]) -> int:

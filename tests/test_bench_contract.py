@@ -87,3 +87,30 @@ def test_mix_probe_reports_a_rate_and_a_plausible_clock(gpu_device):
         omni_attn_capi.mfma_mix_probe(4, 10, sink, None)
     with pytest.raises(RuntimeError):
         omni_attn_capi.mfma_mix_probe(0, 10, sink, torch.zeros(2, dtype=torch.int32, device=gpu_device))
+
+
+@pytest.mark.gpu
+def test_issue_probe_counts_cycles_per_matrix_instruction(gpu_device):
+    """One MFMA alone takes a SIMD 32 cycles; eight v_fma_f32 beside it make the vector pipe the
+    longer one.  Bad arguments are status codes, not launches."""
+    import torch
+
+    import omni_attn_capi
+
+    ticks = torch.zeros(17, dtype=torch.int64, device=gpu_device)
+
+    def cycles(n_plain, n_exp, waves, iters=512):
+        omni_attn_capi.issue_probe(n_plain, n_exp, waves, iters, ticks)
+        torch.cuda.synchronize()
+        t = ticks.tolist()
+        span = max(t[2 * w + 1] for w in range(4 * waves)) - min(t[2 * w] for w in range(4 * waves))
+        return span / (4.0 * iters * waves)
+
+    alone = cycles(0, 0, 2)
+    assert 30.0 < alone < 40.0
+    assert cycles(8, 2, 2) > alone * 1.3
+    for bad in ((3, 0, 2), (0, 3, 2), (0, 0, 3), (10, 0, 1)):
+        with pytest.raises(RuntimeError):
+            omni_attn_capi.issue_probe(bad[0], bad[1], bad[2], 16, ticks)
+    with pytest.raises(RuntimeError):
+        omni_attn_capi.issue_probe(0, 0, 1, 16, torch.zeros(4, dtype=torch.int64, device=gpu_device))
