@@ -48,8 +48,9 @@ struct BwdParams {
   uint16_t* dk;
   uint16_t* dv;
   // workspace [2][B,H,S], written by the dQ kernel and read by the dK/dV kernel: plane 0 is
-  // -delta = -rowsum(dO . O); plane 1 the exponent offset of the row, LSE * log2(e), +inf for a
-  // row without any allowed key or beyond the sequence (every weight of such a row becomes 0)
+  // -delta = -rowsum(dO . O); plane 1 the offset of the row's scores, -LSE * sqrt(D), -inf for a
+  // row without any allowed key or beyond the sequence (every weight of such a row becomes 0) --
+  // or, in the soft-capped instances, the exponent offset LSE * log2(e), +inf for such a row
   float* ws;
   const int32_t* kv_num_blocks;
   const int32_t* kv_indices;
@@ -64,6 +65,12 @@ struct BwdParams {
   float scale;    // 1 / sqrt(D)
   float softcap;  // > 0: the forward replaced x = s / sqrt(D) by softcap * tanh(x / softcap)
   float cap_c2;   // 2 * log2(e) / (sqrt(D) * softcap)
+};
+
+// sqrt(D) for the head dimensions of the instances.
+template <int D>
+struct SqrtOf {
+  static constexpr float value = D == 128 ? 11.313708498984761f : (D == 64 ? 8.f : 5.656854249492381f);
 };
 
 // Weight and score-gradient factor of one score.  Plain: p = exp2(s * sl2 - lse2), factor 1.
@@ -249,10 +256,13 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5, c = lane & 31;
 
+  // Rows at or beyond the sequence are never used: the resources of K and V end there (those
+  // rows arrive as zeros) and the query rows beyond it are replaced by zeros below, whatever the
+  // caller left in the padding.
   const size_t slab = size_t(bh) * size_t(p.S) * D;
-  const uint32_t slab_bytes = uint32_t(p.S) * uint32_t(D * 2);
-  const i32x4_t rK = make_buffer_resource(p.k + slab, slab_bytes);
-  const i32x4_t rV = make_buffer_resource(p.v + slab, slab_bytes);
+  const uint32_t live_bytes = uint32_t(p.seqlen) * uint32_t(D * 2);
+  const i32x4_t rK = make_buffer_resource(p.k + slab, live_bytes);
+  const i32x4_t rV = make_buffer_resource(p.v + slab, live_bytes);
   const int q_row = qb * QB + 32 * w + c;
   const int q_wave_min = qb * QB + 32 * w;
   const int qr = q_row < p.S ? q_row : p.S - 1;
@@ -285,9 +295,11 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
     const uint16_t* op = p.o + slab + size_t(qr) * D + 8 * g;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
-      qf[s] = *reinterpret_cast<const u32x4_t*>(qp + 16 * s);
-      dof[s] = *reinterpret_cast<const u32x4_t*>(dop + 16 * s);
-      const u32x4_t of = *reinterpret_cast<const u32x4_t*>(op + 16 * s);
+      const u32x4_t none4 = {0u, 0u, 0u, 0u};
+      const bool row_in = q_row < p.seqlen;
+      qf[s] = row_in ? *reinterpret_cast<const u32x4_t*>(qp + 16 * s) : none4;
+      dof[s] = row_in ? *reinterpret_cast<const u32x4_t*>(dop + 16 * s) : none4;
+      const u32x4_t of = row_in ? *reinterpret_cast<const u32x4_t*>(op + 16 * s) : none4;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         // (elements are copied to scalars first: a bit cast applied directly to a vector element
@@ -317,7 +329,12 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   const float lse2 = row_live ? lse * 1.4426950408889634f : INFINITY;
   if (q_row < p.S && g == 0) {
     p.ws[size_t(bh) * p.S + q_row] = -delta;
-    p.ws[size_t(p.n_slabs) * p.S + size_t(bh) * p.S + q_row] = lse2;
+    // The dK/dV kernel starts the accumulator of a row's scores at -LSE * sqrt(D), so that the
+    // exponent of a weight is the score times log2(e) / sqrt(D) and nothing else (-inf: every
+    // weight of the row is 0).  A soft-capped score is not linear in the product: there the
+    // plane holds the offset itself.
+    p.ws[size_t(p.n_slabs) * p.S + size_t(bh) * p.S + q_row] =
+        CAP ? lse2 : (row_live ? -lse * SqrtOf<D>::value : -INFINITY);
   }
 
   const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -502,50 +519,93 @@ struct BwdDkdvTraits {
   static constexpr int kKeyGroups = KB / 32;       // 32 keys per wave
   static constexpr int kRoleThreads = KB * 2;      // one wave per key group in each of the two roles
   static constexpr int kThreads = KB * 4;
-  static constexpr int kStep = 32;                 // query rows per step
+  // Query rows per step.  At head_dim 128 with 128-key blocks: 64, worked as two 32-row halves
+  // whose products and vector work overlap inside a wave (one workgroup of eight waves per
+  // compute unit, two waves per SIMD).  Elsewhere 32, so that two workgroups share a compute
+  // unit: a 64-key workgroup has four waves, and at head_dim <= 64 the products of a step are so
+  // short that four waves per SIMD hide more than longer steps gain (measured at head_dim 64:
+  // 64-row steps at two waves per SIMD take 1.3 x the time of 32-row steps at four).
+  static constexpr int kStep = (KB == 128 && D == 128) ? 64 : 32;
+  static constexpr int kSub = kStep / 32;
   static constexpr int kTileElems = kStep * D;
-  static constexpr int kMaxBitmapWords = 4096;     // 64-slot words of the match bitmap
-  // three sets of two tiles (Q, dO); two sets of the weights one role hands to the other (fp32,
-  // [key group][16][64 lanes]) -- the output staging overlaps tiles and weights; -delta and the
-  // exponent offsets of the rows of three steps; per 64-slot word of a slab's metadata the
-  // bitmap of the slots that list this KV block and mode / tile index of the first
+  // three sets of two tiles (Q, dO) -- the output staging overlaps them
   static constexpr size_t kTileBytes = size_t(6) * kTileElems * sizeof(uint16_t);
-  static constexpr size_t kWeightBytes = size_t(2) * kKeyGroups * 16 * 64 * sizeof(float);
-  // (the launch asks for the words its metadata needs, so small problems fit two workgroups)
-  static constexpr size_t lds_bytes(size_t bitmap_words) {
-    return kTileBytes + kWeightBytes + 6 * kStep * sizeof(float) + bitmap_words * (8 + 4);
-  }
+  // the weights one role hands to the other, 16-bit and in B-operand order:
+  // [2 steps in flight][key group][32-row half][2][64 lanes] 16-byte words
+  static constexpr size_t kHandBytes = size_t(2) * kKeyGroups * kSub * 2 * 64 * 16;
+  // -delta and the exponent offsets of the rows of three steps
+  static constexpr size_t kRowBytes = size_t(6) * kStep * sizeof(float);
+  static constexpr size_t kFixedBytes = kTileBytes + kHandBytes + kRowBytes;
+  // per 64-slot word of a slab's metadata: the bitmap of the slots that list this KV block (8
+  // bytes) and mode / tile index of the first (4 bytes).  The launch asks for the words its
+  // metadata needs, so small problems fit two workgroups per compute unit.
+  static constexpr size_t kLdsLimit = size_t(160) * 1024;
+  static constexpr int kMaxBitmapWords =
+      (kLdsLimit - kFixedBytes) / 12 < 4096 ? int((kLdsLimit - kFixedBytes) / 12) : 4096;
+  static constexpr size_t lds_bytes(size_t bitmap_words) { return kFixedBytes + bitmap_words * 12; }
   static constexpr size_t kLdsBytes = lds_bytes(kMaxBitmapWords);
 };
+
+// 64-slot words of match bitmap the dK/dV kernel of a (head_dim, KV block) pair can hold.
+constexpr int bwd_max_bitmap_words(int D, int KB) {
+  return D == 128 ? (KB == 128 ? BwdDkdvTraits<128, 128>::kMaxBitmapWords : BwdDkdvTraits<128, 64>::kMaxBitmapWords)
+       : D == 64  ? (KB == 128 ? BwdDkdvTraits<64, 128>::kMaxBitmapWords : BwdDkdvTraits<64, 64>::kMaxBitmapWords)
+                  : (KB == 128 ? BwdDkdvTraits<32, 128>::kMaxBitmapWords : BwdDkdvTraits<32, 64>::kMaxBitmapWords);
+}
+
+// Two 16-bit values of a word -> fp32 (exact).
+template <bool BF16>
+__device__ __forceinline__ void unpack2(uint32_t w, float& lo, float& hi) {
+  if constexpr (BF16) {
+    const uint32_t l = w << 16, h = w & 0xffff0000u;
+    lo = __builtin_bit_cast(float, l);
+    hi = __builtin_bit_cast(float, h);
+  } else {
+    const f16x2_t v = __builtin_bit_cast(f16x2_t, w);
+    lo = float(v[0]);
+    hi = float(v[1]);
+  }
+}
 
 // One workgroup per KV block, two waves per 32 keys with different work, so that two waves
 // share each SIMD and the vector work of one runs under the matrix work of the other:
 //   the "weight" wave of a key group holds K, computes S = Q.K^T and P for a step, hands P
-//   (times the soft-cap derivative factor, when capped) to its partner through LDS, and
-//   accumulates dV^T += dO^T.P;
+//   (times the soft-cap derivative factor, when capped) to its partner through LDS -- rounded to
+//   16 bits, in the order the partner's product reads it -- and accumulates dV^T += dO^T.P;
 //   the "gradient" wave holds V, computes dP - delta = dO.V^T - delta, and one step later
 //   dS = P (dP - delta) and dK^T += Q^T.dS.
 // The gradient waves run one step behind the weight waves, so one barrier per step orders
 // the hand-over, the tile loads (the weight waves load Q, the gradient waves dO, one step ahead)
 // and the reuse of the three tile sets.
+// A step is kStep query rows.  Its products form one sequence of slots -- first products of the
+// 32-row halves, then second products of the halves -- each slot one MFMA, the LDS fetch of
+// the operand three slots ahead and a share of the vector work of the half whose first
+// product has just finished, with a scheduling fence after each slot: the weights of half u are
+// computed under the products of half u + 1 (or under the second products of half 0).
 template <bool BF16, bool CAP, int D, int QB, int KB>
-__global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(const BwdParams p) {
   using Traits = BwdDkdvTraits<D, KB>;
   constexpr int NKG = Traits::kKeyGroups;
   constexpr int RT = Traits::kRoleThreads;
   constexpr int NW = Traits::kThreads / 64;
   constexpr int STEP = Traits::kStep;
+  constexpr int NSUB = Traits::kSub;
   constexpr int NSTEPS = QB / STEP;  // steps per query block
-  constexpr int NTL = 1;
-  constexpr int KS = D / 16;
+  constexpr int KS = D / 16;         // products of a 32-row half: KS for S (or dP) ...
   constexpr int DT = D / 32;
+  constexpr int NTR = 2 * DT;        // ... and as many for dV^T (or dK^T)
+  constexpr int NS = 2 * NSUB * KS;  // slots of a step
+  constexpr int SPC = 16 / KS;       // scores of a half whose vector work goes beside one product
   constexpr int TILE = Traits::kTileElems;
-  constexpr int NTR = (STEP / 16) * DT;  // fragments of the second product
+  constexpr int PF = 3 < NS ? 3 : NS;  // operand fetch distance in slots
+  constexpr bool PRIO = KB == 64;      // raise the wave priority around the products (it pays
+                                       // with two workgroups per compute unit)
+  static_assert(NTR == KS && QB % STEP == 0 && 16 % KS == 0, "slot layout");
 
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
   uint16_t* const lds16 = reinterpret_cast<uint16_t*>(lds_raw);  // [3 sets][Q, dO][TILE]
-  float* const sW = reinterpret_cast<float*>(lds_raw + Traits::kTileBytes);  // [2 sets][NKG][16][64]
-  float* const sNd = sW + 2 * NKG * 16 * 64;                                 // [3 sets][STEP] -delta
+  uint32_t* const sHand = reinterpret_cast<uint32_t*>(lds_raw + Traits::kTileBytes);
+  float* const sNd = reinterpret_cast<float*>(lds_raw + Traits::kTileBytes + Traits::kHandBytes);  // [3 sets][STEP] -delta
   float* const sL2 = sNd + 3 * STEP;                                         // [3 sets][STEP] exponent offsets
   uint64_t* const sMatch = reinterpret_cast<uint64_t*>(sL2 + 3 * STEP);
   int32_t* const sFirst = reinterpret_cast<int32_t*>(sMatch + p.Tq * ((p.max_blocks + 63) / 64));
@@ -566,26 +626,33 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
   const int rtid = tid - (grad_role ? RT : 0);
   const int g = lane >> 5, c = lane & 31;
 
+  // Rows at or beyond the sequence are never read: the resources of Q and dO end there, so
+  // those rows arrive as zeros whatever the caller left in them.
   const size_t slab = size_t(bh) * size_t(p.S) * D;
-  const uint32_t slab_bytes = uint32_t(p.S) * uint32_t(D * 2);
-  const i32x4_t rQ = make_buffer_resource(p.q + slab, slab_bytes);
-  const i32x4_t rD = make_buffer_resource(p.dout + slab, slab_bytes);
+  const uint32_t live_bytes = uint32_t(p.seqlen) * uint32_t(D * 2);
+  const i32x4_t rQ = make_buffer_resource(p.q + slab, live_bytes);
+  const i32x4_t rD = make_buffer_resource(p.dout + slab, live_bytes);
   const i32x4_t rNd = make_buffer_resource(p.ws + size_t(bh) * p.S, uint32_t(p.S) * 4u);
   const i32x4_t rL2 = make_buffer_resource(p.ws + size_t(p.n_slabs) * p.S + size_t(bh) * p.S, uint32_t(p.S) * 4u);
   const int key_wave_min = kvb * KB + 32 * kg;
   const int key = key_wave_min + c;  // this lane's key row inside the slab
   const int kr = key < p.S ? key : p.S - 1;
+  const bool key_live = key < p.seqlen;
   const bool has_partial = p.partial_idx != nullptr && (p.partial_masks != nullptr || p.partial_bits != nullptr);
   const size_t meta_slab = size_t(bh) * p.Tq;
   const int chunks = (p.max_blocks + 63) / 64;  // 64-slot words per query block
   const int n_words = p.Tq * chunks;
 
-  // This lane's key as B operand: K for a weight wave, V for a gradient wave.
+  // This lane's key as B operand: K for a weight wave, V for a gradient wave (zeros for a key
+  // beyond the sequence).
   u32x4_t bop[KS];
   {
     const uint16_t* src = (grad_role ? p.v : p.k) + slab + size_t(kr) * D + 8 * g;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) bop[s] = *reinterpret_cast<const u32x4_t*>(src + 16 * s);
+    for (int s = 0; s < KS; ++s) {
+      const u32x4_t val = *reinterpret_cast<const u32x4_t*>(src + 16 * s);
+      bop[s] = key_live ? val : u32x4_t{0u, 0u, 0u, 0u};
+    }
   }
 
   // Pass 1: which (query block, slot) pairs list this KV block (after the forward's clamping of
@@ -619,7 +686,6 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
   f32x16_t acc[DT];  // dV^T of a weight wave, dK^T of a gradient wave
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16;
-  const bool key_live = key < p.seqlen;
 
   // Pass 2: the matches in ascending (query block, slot) order, each as NSTEPS steps of STEP
   // query rows, skipping steps beyond the sequence and CAUSAL steps entirely above the diagonal.
@@ -686,9 +752,13 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
     }
   };
   const uint32_t lds_tiles = lds_offset_of(lds16);
-  const uint32_t lds_w = lds_offset_of(sW) + uint32_t(kg) * 4096u + uint32_t(lane) * 16u;
+  const uint32_t hand_lane = lds_offset_of(sHand) + uint32_t(kg) * (NSUB * 2048u) + uint32_t(lane) * 16u;
   const uint32_t lds_nd = lds_offset_of(sNd), lds_l2 = lds_offset_of(sL2);
   auto tile_at = [&](int set, int which) { return lds_tiles + uint32_t(set * 2 + which) * (TILE * 2u); };
+  // the four words of half `half` of 32-row half u of the step with parity par
+  auto hand_at = [&](int par, int u, int half) {
+    return hand_lane + uint32_t(par) * (NKG * NSUB * 2048u) + uint32_t(u) * 2048u + uint32_t(half) * 1024u;
+  };
   // The rows of step j + 1 are loaded during iteration j: Q and the exponent offsets by the
   // weight waves, dO and -delta by the gradient waves.
   auto load_q = [&](const BwdStepInfo& st, int set) {
@@ -704,116 +774,171 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
   const uint32_t row_lane = bwd_row_lane<D>(g, c);
   const uint32_t tr_lo = bwd_tr_lane<D>(g, c, 0), tr_hi = bwd_tr_lane<D>(g, c, 1);
 
-  // Weight wave, one step: S = Q.K^T (lane = key, registers = query rows), P, dV^T += dO^T.P.
-  auto weight_step = [&](int set, int par, uint32_t kw, bool all_allowed) {
-    const uint32_t aQ = tile_at(set, 0) + row_lane, tD0 = tile_at(set, 1) + tr_lo, tD1 = tile_at(set, 1) + tr_hi;
-    u32x4_t fa[KS];
-    static_for<KS>([&](auto ks) {
-      constexpr int s = decltype(ks)::value;
-      fa[s] = lds_b128_at(aQ ^ uint32_t(32 * s));
-    });
-    __builtin_amdgcn_sched_barrier(0);
-    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(1);  // products first (it pays with two workgroups per compute unit)
-    f32x16_t sc = zero16;
-    static_for<KS>([&](auto ks) {
-      constexpr int s = decltype(ks)::value;
-      sc = mfma_32x32x16<BF16>(fa[s], bop[s], sc);
-    });
-    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(0);
-    u32x4_t gd[NTR];
-    static_for<NTR>([&](auto jc) {
-      constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
-      gd[ts * DT + dt] = lds_tr_pair_at((tD0 ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u,
-                                        (tD1 ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u);
-    });
-    f32x4_t l4[4];
-    static_for<4>([&](auto ic) {
-      constexpr int i4 = decltype(ic)::value;
-      // registers 4 i4 .. +3 are query rows 8 i4 + 4 g .. +3 of the step
-      l4[i4] = lds_f32x4_at(lds_l2 + uint32_t(set * STEP + 8 * i4) * 4u + 16u * g);
-    });
-    __builtin_amdgcn_sched_barrier(0);
-    u32x4_t pb[2];
-    auto weights = [&](auto masked_c) {
-      constexpr bool MASKED = decltype(masked_c)::value;
-      static_for<4>([&](auto ic) {
-        constexpr int i4 = decltype(ic)::value;
-        float pv[4];
-        f32x4_t hand;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float wgt, fac;
-          bwd_weight<CAP>(sc[4 * i4 + e], l4[i4][e], p, wgt, fac);
-          if constexpr (MASKED) wgt = ((kw >> (8 * i4 + e)) & 1u) ? wgt : 0.f;  // (kw is already shifted by 4 g)
-          pv[e] = wgt;
-          hand[e] = wgt * fac;
-        }
-        *(__attribute__((address_space(3))) f32x4_t*)(lds_w + uint32_t(par) * (NKG * 4096u) + uint32_t(i4) * 1024u) = hand;
-        pb[i4 >> 1][2 * (i4 & 1) + 0] = pack2<BF16>(pv[0], pv[1]);
-        pb[i4 >> 1][2 * (i4 & 1) + 1] = pack2<BF16>(pv[2], pv[3]);
-      });
-    };
-    if (all_allowed) {  // (wave-uniform) a FULL step whose keys are all inside the sequence needs no mask
-      weights(std::integral_constant<bool, false>{});
+  // Operand n of a step's slot sequence, from the tile read row-wise (first products: rows
+  // 32 u + lane of the tile at k-step s) or transposed (second products: columns 32 dt .. +31
+  // at rows 32 u + 16 ts .. +15).
+  auto operand = [&](auto nc, uint32_t a_rows, uint32_t a_tr0, uint32_t a_tr1) {
+    constexpr int n = decltype(nc)::value;
+    constexpr int ch = n / KS, s = n % KS;
+    if constexpr (ch < NSUB) {
+      return lds_b128_at((a_rows ^ uint32_t(32 * s)) + uint32_t(ch) * (32u * D * 2u));
     } else {
-      weights(std::integral_constant<bool, true>{});
+      constexpr int u = ch - NSUB, ts = s / DT, dt = s % DT;
+      constexpr uint32_t off = uint32_t(2 * u + ts) * (16u * D * 2u);
+      return lds_tr_pair_at((a_tr0 ^ uint32_t(64 * dt)) + off, (a_tr1 ^ uint32_t(64 * dt)) + off);
     }
-    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(1);
-    static_for<NTR>([&](auto jc) {
-      constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
-      acc[dt] = mfma_32x32x16<BF16>(gd[ts * DT + dt], pb[ts], acc[dt]);
+  };
+
+  // Weight wave, one step: S = Q.K^T (lane = key, registers = query rows), P, dV^T += dO^T.P.
+  // The accumulator of a half's scores starts at the rows' offsets -LSE * sqrt(D) -- at -inf where
+  // the step's mask (`masked`, wave-uniform: the words kw are only looked at then) forbids the
+  // pair -- so a weight is exp2(score * sl2) and the mask costs nothing inside the slots.  A
+  // soft-capped score is not linear in the product: there the accumulator starts at zero, the
+  // offsets are fetched when the weights are computed and the mask is applied to the weights.
+  auto weight_step = [&](int set, int par, const uint32_t (&kw)[NSUB], bool masked) {
+    const uint32_t aQ = tile_at(set, 0) + row_lane, tD0 = tile_at(set, 1) + tr_lo, tD1 = tile_at(set, 1) + tr_hi;
+    // The row offsets of the workspace: registers 4 i .. +3 of a half are its query rows
+    // 8 i + 4 g .. +3.
+    auto row_offsets = [&](int u, int i4) {
+      return lds_f32x4_at(lds_l2 + uint32_t(set * STEP + 32 * u + 8 * i4) * 4u + 16u * g);
+    };
+    // 0 or ~0: may register r of half u keep its value?  (kw is already shifted by 4 g: bit
+    // 8 (r / 4) + r % 4 is the row of register r)
+    auto keep_bits = [&](auto uc, auto rc) {
+      constexpr int u = decltype(uc)::value, r = decltype(rc)::value;
+      return uint32_t(__builtin_amdgcn_sbfe(int(kw[u]), 8 * (r >> 2) + (r & 3), 1));
+    };
+    f32x16_t sc[NSUB];
+    u32x4_t pb[NSUB][2];   // P packed to 16 bits, B-operand order
+    u32x4_t hb[NSUB][2];   // what the partner gets when capped: P times the soft-cap factor
+    f32x4_t lq = {0.f, 0.f, 0.f, 0.f};
+    auto weights = [&](auto uc, auto ic) {
+      constexpr int u = decltype(uc)::value, i = decltype(ic)::value;
+      static_for<SPC / 2>([&](auto jc) {
+        constexpr int r = SPC * i + 2 * decltype(jc)::value;
+        float w0, w1;
+        if constexpr (CAP) {
+          float f0, f1;
+          if constexpr ((r & 3) == 0) lq = row_offsets(u, r >> 2);
+          bwd_weight<true>(sc[u][r], lq[r & 3], p, w0, f0);
+          bwd_weight<true>(sc[u][r + 1], lq[(r + 1) & 3], p, w1, f1);
+          const uint32_t b0 = __builtin_bit_cast(uint32_t, w0) & keep_bits(uc, IntC<r>{});
+          const uint32_t b1 = __builtin_bit_cast(uint32_t, w1) & keep_bits(uc, IntC<r + 1>{});
+          w0 = __builtin_bit_cast(float, b0);
+          w1 = __builtin_bit_cast(float, b1);
+          hb[u][r >> 3][(r & 7) >> 1] = pack2<BF16>(w0 * f0, w1 * f1);
+        } else {  // the scores already carry their row's offset and the mask
+          w0 = __builtin_amdgcn_exp2f(sc[u][r] * p.sl2);
+          w1 = __builtin_amdgcn_exp2f(sc[u][r + 1] * p.sl2);
+        }
+        pb[u][r >> 3][(r & 7) >> 1] = pack2<BF16>(w0, w1);
+      });
+      if constexpr (((i + 1) * SPC) % 8 == 0) {  // four words are complete: to the partner
+        constexpr int half = (i + 1) * SPC / 8 - 1;
+        if constexpr (CAP) {
+          *(__attribute__((address_space(3))) u32x4_t*)(hand_at(par, u, half)) = hb[u][half];
+        } else {
+          *(__attribute__((address_space(3))) u32x4_t*)(hand_at(par, u, half)) = pb[u][half];
+        }
+      }
+    };
+    u32x4_t opq[PF];
+    static_for<PF>([&](auto nc) { opq[decltype(nc)::value] = operand(nc, aQ, tD0, tD1); });
+    if constexpr (PRIO) __builtin_amdgcn_s_setprio(1);
+    static_for<NS>([&](auto nc) {
+      constexpr int n = decltype(nc)::value;
+      constexpr int ch = n / KS, s = n % KS;
+      if constexpr (ch < NSUB) {
+        if constexpr (s == 0) {
+          if constexpr (CAP) {
+            sc[ch] = zero16;
+          } else {
+            static_for<4>([&](auto ic) {
+              constexpr int i4 = decltype(ic)::value;
+              const f32x4_t o4 = row_offsets(ch, i4);
+              sc[ch][4 * i4 + 0] = o4[0];
+              sc[ch][4 * i4 + 1] = o4[1];
+              sc[ch][4 * i4 + 2] = o4[2];
+              sc[ch][4 * i4 + 3] = o4[3];
+            });
+            if (masked) {
+              static_for<16>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                const uint32_t keep = keep_bits(IntC<ch>{}, rc);
+                const uint32_t bits = __builtin_bit_cast(uint32_t, float(sc[ch][r]));
+                sc[ch][r] = __builtin_bit_cast(float, (bits & keep) | (0xff800000u & ~keep));
+              });
+            }
+          }
+        }
+        sc[ch] = mfma_32x32x16<BF16>(opq[n % PF], bop[s], sc[ch]);
+      } else {
+        constexpr int u = ch - NSUB, ts = s / DT, dt = s % DT;
+        acc[dt] = mfma_32x32x16<BF16>(opq[n % PF], pb[u][ts], acc[dt]);
+      }
+      if constexpr (n + PF < NS) opq[n % PF] = operand(IntC<n + PF>{}, aQ, tD0, tD1);
+      // the weights of half ch - 1 go beside the products of chain ch
+      if constexpr (NSUB > 1 && ch >= 1 && ch <= NSUB) weights(IntC<ch - 1>{}, IntC<s>{});
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (NSUB == 1 && n == KS - 1) {  // a one-half step: nothing to put them under
+        if constexpr (PRIO) __builtin_amdgcn_s_setprio(0);
+        static_for<KS>([&](auto ic) { weights(IntC<0>{}, ic); });
+        if constexpr (PRIO) __builtin_amdgcn_s_setprio(1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     });
-    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(0);
+    if constexpr (PRIO) __builtin_amdgcn_s_setprio(0);
   };
   // Gradient wave, one step: dP - delta = dO.V^T - delta (the accumulator starts at -delta),
   // dS = P (dP - delta) with the partner's P, dK^T += Q^T.dS.
   auto grad_step = [&](int set, int par) {
     const uint32_t aD = tile_at(set, 1) + row_lane, tQ0 = tile_at(set, 0) + tr_lo, tQ1 = tile_at(set, 0) + tr_hi;
-    f32x16_t dp;
-    static_for<4>([&](auto ic) {
-      constexpr int i4 = decltype(ic)::value;
-      const f32x4_t nd = lds_f32x4_at(lds_nd + uint32_t(set * STEP + 8 * i4) * 4u + 16u * g);
-      dp[4 * i4 + 0] = nd[0];
-      dp[4 * i4 + 1] = nd[1];
-      dp[4 * i4 + 2] = nd[2];
-      dp[4 * i4 + 3] = nd[3];
+    f32x16_t dp[NSUB];
+    u32x4_t hand[NSUB][2], dsb[NSUB][2];
+    static_for<4 * NSUB>([&](auto ic) {
+      constexpr int u = decltype(ic)::value / 4, i4 = decltype(ic)::value % 4;
+      const f32x4_t nd = lds_f32x4_at(lds_nd + uint32_t(set * STEP + 32 * u + 8 * i4) * 4u + 16u * g);
+      dp[u][4 * i4 + 0] = nd[0];
+      dp[u][4 * i4 + 1] = nd[1];
+      dp[u][4 * i4 + 2] = nd[2];
+      dp[u][4 * i4 + 3] = nd[3];
     });
-    u32x4_t fb[KS];
-    static_for<KS>([&](auto ks) {
-      constexpr int s = decltype(ks)::value;
-      fb[s] = lds_b128_at(aD ^ uint32_t(32 * s));
+    auto score_grads = [&](auto uc, auto ic) {
+      constexpr int u = decltype(uc)::value, i = decltype(ic)::value;
+      static_for<SPC / 2>([&](auto jc) {
+        constexpr int r = SPC * i + 2 * decltype(jc)::value;
+        float h0, h1;
+        unpack2<BF16>(hand[u][r >> 3][(r & 7) >> 1], h0, h1);
+        dsb[u][r >> 3][(r & 7) >> 1] = pack2<BF16>(h0 * dp[u][r], h1 * dp[u][r + 1]);
+      });
+    };
+    u32x4_t opq[PF];
+    static_for<PF>([&](auto nc) { opq[decltype(nc)::value] = operand(nc, aD, tQ0, tQ1); });
+    if constexpr (PRIO) __builtin_amdgcn_s_setprio(1);
+    static_for<NS>([&](auto nc) {
+      constexpr int n = decltype(nc)::value;
+      constexpr int ch = n / KS, s = n % KS;
+      if constexpr (ch < NSUB) {
+        if constexpr (s == 0) {
+          hand[ch][0] = lds_b128_at(hand_at(par, ch, 0));
+          hand[ch][1] = lds_b128_at(hand_at(par, ch, 1));
+        }
+        dp[ch] = mfma_32x32x16<BF16>(opq[n % PF], bop[s], dp[ch]);
+      } else {
+        constexpr int u = ch - NSUB, ts = s / DT, dt = s % DT;
+        acc[dt] = mfma_32x32x16<BF16>(opq[n % PF], dsb[u][ts], acc[dt]);
+      }
+      if constexpr (n + PF < NS) opq[n % PF] = operand(IntC<n + PF>{}, aD, tQ0, tQ1);
+      if constexpr (NSUB > 1 && ch >= 1 && ch <= NSUB) score_grads(IntC<ch - 1>{}, IntC<s>{});
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (NSUB == 1 && n == KS - 1) {
+        if constexpr (PRIO) __builtin_amdgcn_s_setprio(0);
+        static_for<KS>([&](auto ic) { score_grads(IntC<0>{}, ic); });
+        if constexpr (PRIO) __builtin_amdgcn_s_setprio(1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     });
-    __builtin_amdgcn_sched_barrier(0);
-    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(1);
-    static_for<KS>([&](auto ks) {
-      constexpr int s = decltype(ks)::value;
-      dp = mfma_32x32x16<BF16>(fb[s], bop[s], dp);
-    });
-    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(0);
-    u32x4_t gq[NTR];
-    static_for<NTR>([&](auto jc) {
-      constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
-      gq[ts * DT + dt] = lds_tr_pair_at((tQ0 ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u,
-                                        (tQ1 ^ uint32_t(64 * dt)) + uint32_t(ts) * 16u * D * 2u);
-    });
-    f32x4_t hand[4];
-    static_for<4>([&](auto ic) {
-      constexpr int i4 = decltype(ic)::value;
-      hand[i4] = lds_f32x4_at(lds_w + uint32_t(par) * (NKG * 4096u) + uint32_t(i4) * 1024u);
-    });
-    __builtin_amdgcn_sched_barrier(0);
-    u32x4_t dsb[2];
-    static_for<4>([&](auto ic) {
-      constexpr int i4 = decltype(ic)::value;
-      dsb[i4 >> 1][2 * (i4 & 1) + 0] = pack2<BF16>(hand[i4][0] * dp[4 * i4 + 0], hand[i4][1] * dp[4 * i4 + 1]);
-      dsb[i4 >> 1][2 * (i4 & 1) + 1] = pack2<BF16>(hand[i4][2] * dp[4 * i4 + 2], hand[i4][3] * dp[4 * i4 + 3]);
-    });
-    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(1);
-    static_for<NTR>([&](auto jc) {
-      constexpr int ts = decltype(jc)::value / DT, dt = decltype(jc)::value % DT;
-      acc[dt] = mfma_32x32x16<BF16>(gq[ts * DT + dt], dsb[ts], acc[dt]);
-    });
-    if constexpr (KB == 64) __builtin_amdgcn_s_setprio(0);
+    if constexpr (PRIO) __builtin_amdgcn_s_setprio(0);
   };
 
   // Bits of one partial tile for this lane's key: bit j = query row q_local0 + j of the tile
@@ -850,17 +975,22 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
     }
     for (int j = 0; cur.valid || prev.valid; ++j) {
       const BwdStepInfo nxt = cur.valid ? next_step() : none;
-      // mask word of this lane's key: bit i = query row row0 + i attends it
-      uint32_t kw = 0;
+      // mask words of this lane's key: bit i of word u = query row row0 + 32 u + i attends it
+      uint32_t kw[NSUB];
+#pragma unroll
+      for (int u = 0; u < NSUB; ++u) kw[u] = 0;
       if constexpr (!GRAD) {
         if (cur.valid) {
-          uint32_t m = key_live ? 0xffffffffu : 0u;
-          if (cur.mode == kCausal) {  // rows at or after the key
-            const int n = key - cur.row0;
-            m &= n <= 0 ? 0xffffffffu : (n >= 32 ? 0u : (0xffffffffu << (n & 31)));
+#pragma unroll
+          for (int u = 0; u < NSUB; ++u) {
+            uint32_t m = key_live ? 0xffffffffu : 0u;
+            if (cur.mode == kCausal) {  // rows at or after the key
+              const int n = key - (cur.row0 + 32 * u);
+              m &= n <= 0 ? 0xffffffffu : (n >= 32 ? 0u : (0xffffffffu << (n & 31)));
+            }
+            if (cur.mode == kPartial) m &= partial_column(cur.pid, cur.row0 + 32 * u - cur.blk * QB);
+            kw[u] = m >> (4 * g);
           }
-          if (cur.mode == kPartial) m &= partial_column(cur.pid, cur.row0 - cur.blk * QB);
-          kw = m >> (4 * g);
         }
       }
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the tile this wave loaded has landed
@@ -868,7 +998,10 @@ __global__ void __launch_bounds__(KB * 4, 1) bwd_dkdv_kernel(const BwdParams p) 
                         // about to be overwritten (step j - 2) is no longer read
       if constexpr (!GRAD) {
         if (nxt.valid) load_q(nxt, s_nxt);
-        if (cur.valid) weight_step(s_cur, j & 1, kw, cur.mode == kFull && key_wave_min + 32 <= p.seqlen);
+        if (cur.valid) {
+          // (wave-uniform) a FULL step whose keys are all inside the sequence needs no mask
+          weight_step(s_cur, j & 1, kw, !(cur.mode == kFull && key_wave_min + 32 <= p.seqlen));
+        }
       } else {
         if (nxt.valid) load_do(nxt, s_nxt);
         if (prev.valid) grad_step(s_prev, (j + 1) & 1);

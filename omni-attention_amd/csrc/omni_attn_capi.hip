@@ -234,7 +234,7 @@ int backward(const void* q, const void* k, const void* v, const void* o, const v
       total * max_blocks > (1LL << 40) || (long long)num_partial * QB * KB > 0x7fffffffLL * 64)
     return OMNI_ATTN_ERR_TOO_LARGE;
   // the dK/dV kernel keeps one bit per (query block, slot) of a slab in LDS
-  if ((long long)Tq * ((max_blocks + 63) / 64) > BwdDkdvTraits<128, 128>::kMaxBitmapWords)
+  if ((long long)Tq * ((max_blocks + 63) / 64) > bwd_max_bitmap_words(D, KB))
     return OMNI_ATTN_ERR_TOO_LARGE;
 
   BwdParams p;

@@ -324,10 +324,13 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
   const int g = lane >> 5;
   const int c = lane & 31;
 
+  // Rows at or beyond the sequence are never used: the resources of K and V end there (those
+  // rows arrive as zeros) and the query rows beyond it are replaced by zeros, whatever the caller
+  // left in the padding.
   const size_t slab = size_t(bh) * size_t(p.S) * D;
-  const uint32_t slab_bytes = uint32_t(p.S) * uint32_t(D * 2);
-  const i32x4_t rK = make_buffer_resource(p.k + slab, slab_bytes);
-  const i32x4_t rV = make_buffer_resource(p.v + slab, slab_bytes);
+  const uint32_t live_bytes = uint32_t(p.seqlen) * uint32_t(D * 2);
+  const i32x4_t rK = make_buffer_resource(p.k + slab, live_bytes);
+  const i32x4_t rV = make_buffer_resource(p.v + slab, live_bytes);
 
   const int q_row = qb * QB + 32 * w + c;  // this lane's query row inside the slab
   const int q_wave_min = qb * QB + 32 * w;
@@ -368,7 +371,8 @@ __global__ void __launch_bounds__(QB * 2, 2) fwd_kernel(const FwdParams p) {
     const int qr = q_row < p.S ? q_row : p.S - 1;
     const uint16_t* qp = p.q + slab + size_t(qr) * D + 8 * g;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const u32x4_t*>(qp + 16 * s);
+    for (int s = 0; s < KS; ++s)
+      qf[s] = q_row < p.seqlen ? *reinterpret_cast<const u32x4_t*>(qp + 16 * s) : u32x4_t{0u, 0u, 0u, 0u};
   }
   // Step `it` (clamped to the last step of the walk; steps past the end are only ever
   // used as the address of a tile load whose data nobody reads).
