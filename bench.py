@@ -14,6 +14,9 @@ time that ramp instead of the kernel.  K and W are exactly what was passed.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
     python bench.py --sweep-bands     # runtime against the number of listed blocks (fixed shape)
+Extra fields of the line: `from_idle` (the same K steps with no settle phase), `operator` (host time
+per call of the Python operator next to the bare C-ABI call and the kernel), `c2_interleaved_8k`,
+`c2_interleaved_backward`.
     python bench.py --kernel-source-hash   # hash that ties a traffic measurement to the kernel sources
 """
 import argparse
@@ -210,194 +213,6 @@ def band_sweep(dev, steps, warmup):
     }
 
 
-def fixed_cost_study(dev, seed, steps, warmup):
-    """Where the time of c2_interleaved goes besides the per-block work: the same launch with
-    every list repeated 2x and 3x (same workgroups, 2x / 3x the steps: r*T1 - Tr is r - 1 times the
-    part that does not grow with the lists), with all block types FULL (no mask work), with the
-    same number of blocks spread evenly over the query blocks (no imbalance), and the dense and
-    plain causal controls of the same shape.  Kernel times are medians of HIP-event brackets."""
-    import torch
-
-    import omni_attn_capi
-    from baseline_configs import make_workload
-
-    w = make_workload("c2_interleaved", seed=seed)
-    m = w.block_mask
-    B, H, S, D = w.q.shape
-    QB, KB = m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE
-    q, k, v = (t.to(dev) for t in (w.q, w.k, w.v))
-    o = torch.empty_like(q)
-    lse = torch.empty(B, H, S, dtype=torch.float32, device=dev)
-    stream = torch.cuda.current_stream(dev)
-    per_block = 4.0 * QB * KB * D
-    nb0, idx0, tys0 = m.kv_num_blocks, m.kv_indices, m.block_mask_types
-    Tq, MB = nb0.shape[2], idx0.shape[3]
-
-    def run(nb, idx, tys, what):
-        nbd, idxd, tysd = (t.to(dev).contiguous() for t in (nb, idx, tys))
-
-        def step():
-            omni_attn_capi.fwd(q, k, v, o, lse, nbd, idxd, tysd, QB, KB, S, None, None, stream=stream.cuda_stream)
-
-        for _ in range(warmup):
-            step()
-        torch.cuda.synchronize()
-        st = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-        en = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-        for i in range(steps):
-            st[i].record(stream)
-            step()
-            en[i].record(stream)
-        torch.cuda.synchronize()
-        ms = statistics.median(a.elapsed_time(b) for a, b in zip(st, en))
-        blocks = int(nb.sum().item())
-        return {"case": what, "listed_blocks": blocks, "kernel_us": ms * 1e3,
-                "tflops": per_block * blocks / (ms * 1e-3) / 1e12, "ns_per_block": ms * 1e6 / blocks}
-
-    t_end = time.perf_counter() + 0.25  # settle the clock under this load
-    nbd, idxd, tysd = (t.to(dev) for t in (nb0, idx0, tys0))
-    while time.perf_counter() < t_end:
-        for _ in range(10):
-            omni_attn_capi.fwd(q, k, v, o, lse, nbd, idxd, tysd, QB, KB, S, None, None, stream=stream.cuda_stream)
-        torch.cuda.synchronize()
-    rows = [run(nb0, idx0, tys0, "c2_interleaved as it is")]
-    T1 = rows[0]["kernel_us"]
-    ar = torch.arange(MB * 3)
-    for r in (2, 3):
-        idx = torch.zeros(B, H, Tq, MB * r, dtype=torch.int32)
-        tys = torch.zeros(B, H, Tq, MB * r, dtype=torch.int32)
-        for b in range(B):
-            src = (ar[: MB * r].view(1, -1) % nb0[b, 0].clamp(min=1).view(-1, 1)).long()
-            idx[b] = torch.gather(idx0[b, 0], 1, src).unsqueeze(0).expand(H, -1, -1)
-            tys[b] = torch.gather(tys0[b, 0], 1, src).unsqueeze(0).expand(H, -1, -1)
-        row = run(nb0 * r, idx, tys, f"every list repeated {r}x")
-        row["fixed_us_estimate"] = (r * T1 - row["kernel_us"]) / (r - 1)
-        rows.append(row)
-    rows.append(run(nb0, idx0, torch.where(tys0 == 1, torch.full_like(tys0, 2), tys0), "all listed blocks FULL"))
-    tot = int(nb0.sum().item())
-    per = tot // (B * H * Tq)
-    nbb = torch.full((B, H, Tq), per, dtype=torch.int32)
-    nbb.view(-1)[: tot - per * B * H * Tq] += 1
-    idxb = torch.arange(MB, dtype=torch.int32).expand(B, H, Tq, MB).contiguous()
-    tysb = torch.full((B, H, Tq, MB), 2, dtype=torch.int32)
-    rows.append(run(nbb, idxb, tysb, "same total, spread evenly over the query blocks"))
-    rows.append(run(torch.full((B, H, Tq), MB, dtype=torch.int32), idxb, tysb, "dense control"))
-    nbc = (torch.arange(Tq, dtype=torch.int32) + 1).expand(B, H, Tq).contiguous()
-    tysc = tysb.clone()
-    for i in range(Tq):
-        tysc[:, :, i, i] = 1
-    rows.append(run(nbc, idxb, tysc, "plain causal"))
-    return {"study": "c2_interleaved: fixed cost, mask cost, imbalance (B=2 H=32 S=4096 D=128 bf16, 128/128)",
-            "rows": rows}
-
-
-def power_study(dev, seed, steps, warmup):
-    """What the clock does to the figures.  (1) The library's matrix-instruction loop with eight
-    operand sets, alone and with the forward kernel's LDS operand reads and softmax vector work
-    beside it: rate and the shader clock one of its waves saw.  (2) The forward kernel on
-    c2_interleaved with its real operands, with V zero and with all operands zero: the same
-    instructions in the same order, but matrix cores and data paths that toggle fewer bits draw less
-    power and the device grants a higher clock."""
-    import torch
-
-    import omni_attn_capi
-    from baseline_configs import make_workload
-
-    stream = torch.cuda.current_stream(dev)
-    sink = torch.zeros(1, dtype=torch.float32, device=dev)
-    ticks = torch.zeros(2, dtype=torch.int64, device=dev)
-    names = {0: "mfma only, eight operand sets in turn", 1: "mfma + A operand from LDS",
-             2: "mfma + softmax vector work", 3: "mfma + A operand from LDS + softmax vector work"}
-    mixes = []
-    for mix in range(4):
-        iters = 20000
-        t_end = time.perf_counter() + 0.25
-        while time.perf_counter() < t_end:
-            for _ in range(3):
-                omni_attn_capi.mfma_mix_probe(mix, iters, sink, None, stream.cuda_stream)
-            torch.cuda.synchronize()
-        best = None
-        for _ in range(3):
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record(stream)
-            flops = omni_attn_capi.mfma_mix_probe(mix, iters, sink, ticks, stream.cuda_stream)
-            b.record(stream)
-            torch.cuda.synchronize()
-            tf = flops / (a.elapsed_time(b) * 1e-3) / 1e12
-            cyc, rt = (int(x) for x in ticks.tolist())
-            if best is None or tf > best["tflops"]:
-                best = {"mix": names[mix], "tflops": tf, "shader_clock_mhz": 100.0 * cyc / max(rt, 1),
-                        "frac_of_rated_peak": tf / MFMA_PEAK_TFLOPS}
-        best["mfma_busy_at_that_clock"] = best["tflops"] / (MFMA_PEAK_TFLOPS * best["shader_clock_mhz"] / 2400.0)
-        mixes.append(best)
-
-    w = make_workload("c2_interleaved", seed=seed)
-    m = w.block_mask
-    B, H, S, D = w.q.shape
-    nb, idx, tys = (t.to(dev) for t in (m.kv_num_blocks, m.kv_indices, m.block_mask_types))
-    o = torch.empty(w.q.shape, dtype=w.dtype, device=dev)
-    lse = torch.empty(B, H, S, dtype=torch.float32, device=dev)
-    rows = []
-    for what in ("operands as in the benchmark (standard normal)", "V zero", "Q, K and V zero"):
-        q, k, v = (t.to(dev) for t in (w.q, w.k, w.v))
-        if what != "operands as in the benchmark (standard normal)":
-            v = torch.zeros_like(v)
-        if what == "Q, K and V zero":
-            q, k = torch.zeros_like(q), torch.zeros_like(k)
-
-        def step():
-            omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, None, None,
-                               stream=stream.cuda_stream)
-
-        t_end = time.perf_counter() + 0.25
-        while time.perf_counter() < t_end:
-            for _ in range(10):
-                step()
-            torch.cuda.synchronize()
-        st = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-        en = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-        for i in range(steps):
-            st[i].record(stream)
-            step()
-            en[i].record(stream)
-        torch.cuda.synchronize()
-        ms = statistics.median(a.elapsed_time(b) for a, b in zip(st, en))
-        tf = w.effective_flops / (ms * 1e-3) / 1e12
-        rows.append({"operands": what, "kernel_us": ms * 1e3, "tflops": tf, "frac_of_rated_peak": tf / MFMA_PEAK_TFLOPS})
-    return {"study": "clock under load: instruction mixes of the probe loop, and the forward kernel on "
-                     "c2_interleaved (B=2 H=32 S=4096 D=128 bf16) with operands that toggle fewer bits",
-            "probe_mixes": mixes, "forward_c2_interleaved": rows}
-
-
-def issue_study(dev):
-    """How much softmax vector work fits under a matrix instruction on one SIMD: the issue probe
-    (one workgroup on one compute unit; groups of one bf16 32x32x16 MFMA + n v_fma_f32 + e v_exp_f32
-    on registers of their own) at one and two waves per SIMD.  Cycles per group and SIMD; a matrix
-    instruction alone takes 32."""
-    import torch
-
-    import omni_attn_capi
-
-    ticks = torch.zeros(17, dtype=torch.int64, device=dev)
-    iters = 2048
-    rows = []
-    for n_exp in (0, 1, 2):
-        for n_plain in (0, 2, 4, 6, 8):
-            row = {"v_fma_f32_per_mfma": n_plain, "v_exp_f32_per_mfma": n_exp}
-            for waves in (1, 2):
-                best = None
-                for _ in range(3):
-                    omni_attn_capi.issue_probe(n_plain, n_exp, waves, iters, ticks)
-                    torch.cuda.synchronize()
-                    t = ticks.tolist()
-                    span = max(t[2 * w + 1] for w in range(4 * waves)) - min(t[2 * w] for w in range(4 * waves))
-                    cyc = span / (4.0 * iters * waves)
-                    best = cyc if best is None else min(best, cyc)
-                row["cycles_per_group_per_simd_%dw" % waves] = best
-            rows.append(row)
-    return {"study": "vector work beside the matrix instructions of one SIMD (issue probe)", "rows": rows}
-
-
 def extra_workload(name, seed, dev, steps, warmup, backward=False, settle_ms=150.0):
     """Kernel time of another workload, or of the backward of a workload (HIP events on the launch
     stream, after `settle_ms` of the same load)."""
@@ -459,6 +274,60 @@ def extra_workload(name, seed, dev, steps, warmup, backward=False, settle_ms=150
     return out
 
 
+def operator_overhead(name, seed, dev, calls=200):
+    """What the operator level adds to a launch: host time per call of omni_attention_shared_kv_swizzle
+    (wrapper + module `omni_attn` + C ABI; the mask already on the GPU) and of the bare C-ABI call
+    with preallocated output, both as the wall time of `calls` back-to-back asynchronous calls between
+    two synchronisations, next to the kernel's own duration (HIP events)."""
+    import torch
+
+    import omni_attn_capi
+    import omni_attn_torch
+    from baseline_configs import make_workload
+
+    w = make_workload(name, seed=seed)
+    m = w.block_mask.to(dev)
+    B, H, S, D = w.q.shape
+    q, k, v = (t.to(dev) for t in (w.q, w.k, w.v))
+    o = torch.empty_like(q)
+    stream = torch.cuda.current_stream(dev)
+
+    def op():
+        return omni_attn_torch.omni_attention_shared_kv_swizzle(q, k, v, m)
+
+    def capi():
+        omni_attn_capi.fwd(q, k, v, o, None, m.kv_num_blocks, m.kv_indices, m.block_mask_types, m.Q_BLOCK_SIZE,
+                           m.KV_BLOCK_SIZE, S, m.partial_block_mask_indices, m.partial_block_masks,
+                           stream=stream.cuda_stream)
+
+    def wall(fn):
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(calls):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / calls * 1e3
+
+    t_end = time.perf_counter() + 0.1
+    while time.perf_counter() < t_end:
+        for _ in range(10):
+            capi()
+        torch.cuda.synchronize()
+    op_ms, capi_ms = wall(op), wall(capi)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record(stream)
+    for _ in range(calls):
+        capi()
+    b.record(stream)
+    torch.cuda.synchronize()
+    kernel_ms = a.elapsed_time(b) / calls
+    return {"operator_ms_per_call": op_ms, "capi_ms_per_call": capi_ms, "kernel_ms": kernel_ms,
+            "operator_minus_kernel_us": (op_ms - kernel_ms) * 1e3,
+            "what": "omni_attention_shared_kv_swizzle(query, key, value, block_mask) vs omni_attn_fwd_gfx950"}
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -468,7 +337,8 @@ def main(argv=None):
                     help="keep the GPU under the benchmark's own load for this long before the warm-up "
                          "launches (from idle the shader clock needs some tens of milliseconds to settle)")
     ap.add_argument("--no-extras", action="store_true",
-                    help="skip the measured MFMA peak, the c2_interleaved_8k figure and the backward figure")
+                    help="skip the measured MFMA peak, the c2_interleaved_8k figure, the backward figure and "
+                         "the operator-level timing")
     ap.add_argument("--kernel-source-hash", action="store_true", help="print the hash and exit")
     ap.add_argument("--backward", action="store_true",
                     help="time the backward (dQ kernel + dK/dV kernel) instead of the forward; effective "
@@ -483,16 +353,6 @@ def main(argv=None):
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, so that a counter run of this "
                          "command shows what FETCH_SIZE / WRITE_SIZE read for a known traffic")
-    ap.add_argument("--fixed-cost", action="store_true",
-                    help="instead of the workload: c2_interleaved with its lists repeated, its types all "
-                         "FULL, its blocks spread evenly (fixed cost / mask cost / imbalance of a launch)")
-    ap.add_argument("--power-study", action="store_true",
-                    help="instead of the workload: the probe loop with the forward kernel's LDS reads and "
-                         "vector work beside the matrix instructions (rate and shader clock), and the forward "
-                         "kernel with zero operands")
-    ap.add_argument("--issue-study", action="store_true",
-                    help="instead of the workload: cycles per matrix instruction and SIMD with 0..8 plain and "
-                         "0..2 transcendental vector instructions issued beside each (one compute unit)")
     ap.add_argument("--sweep-bands", action="store_true",
                     help="instead of the workload: kernel time against the number of listed blocks")
     args = ap.parse_args(argv)
@@ -517,15 +377,6 @@ def main(argv=None):
     omni_attn_capi.load_library()  # fail loudly when the HIP library is missing
     if args.sweep_bands:
         print(json.dumps(band_sweep(dev, min(args.steps, 30), min(args.warmup, 5))))
-        return 0
-    if args.issue_study:
-        print(json.dumps(issue_study(dev)))
-        return 0
-    if args.power_study:
-        print(json.dumps(power_study(dev, args.seed, min(args.steps, 60), min(args.warmup, 10))))
-        return 0
-    if args.fixed_cost:
-        print(json.dumps(fixed_cost_study(dev, args.seed, min(args.steps, 60), min(args.warmup, 10))))
         return 0
 
     w = make_workload(args.workload, seed=args.seed)
@@ -585,6 +436,26 @@ def main(argv=None):
             omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, pidx, pm,
                                stream=stream.cuda_stream)
 
+    def timed_steps(n):
+        """Wall time of exactly n launches between two synchronisations (nothing else is enqueued or
+        recorded inside the region)."""
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(n):
+            step()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t
+
+    # From idle: W warm-up launches and K timed ones straight after the uploads, before the GPU has
+    # been under load for any length of time (the shader clock is still settling: reported beside the
+    # headline, never as `value`).
+    from_idle = None
+    if args.clock_settle_ms > 0:
+        for _ in range(args.warmup):
+            step()
+        wall_idle = timed_steps(args.steps)
+        from_idle = {"ms_per_step": wall_idle / args.steps * 1e3, "steps": args.steps, "warmup": args.warmup}
+
     # clock settle: the same launches, for a fixed time, not counted as warm-up or steps
     settle_launches = 0
     t_settle = time.perf_counter()
@@ -597,20 +468,17 @@ def main(argv=None):
 
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
-
-    # timed region: exactly K steps, synchronised on both sides; events on the launch stream
-    # bracket every launch so that the kernel's own duration is measured in the same region
+    # timed region: exactly K bare launches, synchronised on both sides
+    wall = timed_steps(args.steps)
+    # the kernel's own duration: a second pass of the same K launches, each bracketed by events on
+    # the launch stream (kept out of the host-timed region: two event records cost about 6 us a step)
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
     for i in range(args.steps):
         starts[i].record(stream)
         step()
         ends[i].record(stream)
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
 
     if args.calibrate_copy:
         src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
@@ -649,6 +517,9 @@ def main(argv=None):
             "effective_gflop_per_step": flops / 1e9,
         },
         "clock_settle": {"ms": settle_ms, "launches": settle_launches},
+        "from_idle": None if from_idle is None else dict(
+            from_idle, value=flops / (from_idle["ms_per_step"] * 1e-3) / 1e12,
+            note="the same K steps after the same W warm-ups with no clock-settle phase before them"),
         "pct_of_mfma_peak": 100.0 * value / MFMA_PEAK_TFLOPS,
         "kernel_ms_median": med_kernel_ms,
         "roofline": {
@@ -678,6 +549,7 @@ def main(argv=None):
             if not args.backward:
                 out["c2_interleaved_backward"] = extra_workload("c2_interleaved", args.seed, dev,
                                                                 steps=min(args.steps, 50), warmup=5, backward=True)
+        out["operator"] = {name: operator_overhead(name, args.seed, dev) for name in ("c1_causal", "c2_interleaved")}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, args.cpu_budget_s)
     print(json.dumps(out))

@@ -231,40 +231,14 @@ int omni_attn_bwd_noalloc_gfx950(const void* q, const void* k, const void* v, co
 int omni_attn_mfma_peak_probe_gfx950(int dtype, int iters, float* sink, double* flops_out,
                                      void* stream);
 
-/*
- * Measurement aid (no counterpart in the reference): the same bf16 loop with eight operand sets
- * in turn and, by the bits of `mix`, the forward kernel's other work beside the matrix
- * instructions: 1 = the A operand of every instruction is read from LDS (1 KiB per wave and
- * instruction), 2 = the vector work of a softmax (per instruction one fma, exp2 and add, per two
- * a max3 and a 16-bit pack).  No barriers, tile loads or bookkeeping: rate and clock of such a
- * loop show what each kind of work costs beside the matrix instructions.
- * `ticks` (device memory, two 64-bit words, may be NULL) receives from one wave the shader
- * cycles and the 100 MHz real-time ticks its loop took: their ratio x 100 is the shader clock
- * in MHz under this load.  Allocates nothing.
- */
-int omni_attn_mfma_mix_probe_gfx950(int mix, int iters, float* sink, unsigned long long* ticks,
-                                    double* flops_out, void* stream);
-
-/*
- * Measurement aid (no counterpart in the reference): one workgroup on one compute unit,
- * `waves_per_simd` (1 or 2) waves on every SIMD, each running `iters` x 4 groups of one bf16
- * 32x32x16 matrix instruction followed by `n_plain` (0, 2, 4, 6 or 8) v_fma_f32 and `n_exp`
- * (0, 1 or 2) v_exp_f32 on registers of their own.  `ticks` (device memory, at least 17 64-bit
- * words) receives for wave w the shader cycle counter at the start (word 2w) and the end (word
- * 2w + 1) of its loop: (latest end - earliest start) / (4 * iters * waves_per_simd) is the time
- * one SIMD needs per group -- how much vector work fits under a matrix instruction.
- * Allocates nothing.
- */
-int omni_attn_issue_probe_gfx950(int n_plain, int n_exp, int waves_per_simd, int iters,
-                                 unsigned long long* ticks, void* stream);
-
 /* Static description of a return code (never NULL). */
 const char* omni_attn_status_string(int status);
 
 /* hipError_t of the most recent failed launch on the calling thread (0 if none). */
 int omni_attn_last_hip_error(void);
 
-/* Version of this ABI; bumped when a signature changes (2: num_partial added; 3: softcap added). */
+/* Version of this ABI; bumped when a signature changes (2: num_partial added; 3: softcap added;
+ * 4: the two study probes omni_attn_mfma_mix_probe_gfx950 / omni_attn_issue_probe_gfx950 removed). */
 int omni_attn_abi_version(void);
 
 #ifdef __cplusplus

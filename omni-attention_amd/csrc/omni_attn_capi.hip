@@ -31,6 +31,9 @@ template <> int launch_bwd_blocks<true, 128>(const BwdParams&, int, int, hipStre
 
 namespace {
 thread_local int g_last_hip_error = 0;
+}  // namespace
+void omni_attn::record_hip_error(int hip_error) { g_last_hip_error = hip_error; }
+namespace {
 
 // What the work order needs to know about the device, queried once per device: the number
 // of XCDs (each has its own L2; workgroup ids are dealt round-robin over them), the compute
@@ -385,4 +388,4 @@ extern "C" const char* omni_attn_status_string(int status) {
 
 extern "C" int omni_attn_last_hip_error(void) { return g_last_hip_error; }
 
-extern "C" int omni_attn_abi_version(void) { return 3; }
+extern "C" int omni_attn_abi_version(void) { return 4; }

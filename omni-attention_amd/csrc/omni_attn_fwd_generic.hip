@@ -15,6 +15,12 @@
 
 #include <cmath>
 
+namespace omni_attn {
+// Keeps the hipError_t behind an OMNI_ATTN_ERR_LAUNCH for omni_attn_last_hip_error() (defined
+// beside that function).
+void record_hip_error(int hip_error);
+}  // namespace omni_attn
+
 namespace {
 
 enum : int { kMasked = 0, kCausal = 1, kFull = 2, kPartial = 3 };
@@ -246,8 +252,11 @@ extern "C" int omni_attn_fwd_generic_gfx950(const void* q, const void* k, const 
   const void* kern = dtype == OMNI_ATTN_DTYPE_BF16 ? reinterpret_cast<const void*>(fwd_generic_kernel<true>)
                                                    : reinterpret_cast<const void*>(fwd_generic_kernel<false>);
   void* args[] = {&p};
-  if (hipLaunchKernel(kern, dim3(grid), dim3(64 * kRowsPerWorkgroup), args, 0, static_cast<hipStream_t>(stream)) !=
-      hipSuccess)
+  const hipError_t e = hipLaunchKernel(kern, dim3(grid), dim3(64 * kRowsPerWorkgroup), args, 0,
+                                       static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) {
+    omni_attn::record_hip_error(int(e));
     return OMNI_ATTN_ERR_LAUNCH;
+  }
   return OMNI_ATTN_OK;
 }

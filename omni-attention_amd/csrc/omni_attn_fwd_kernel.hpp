@@ -52,6 +52,10 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
 
 enum : int { kMasked = 0, kCausal = 1, kFull = 2, kPartial = 3 };
 
+// The hipError_t of the last HIP call of this thread that made an entry point return
+// OMNI_ATTN_ERR_LAUNCH (read back through omni_attn_last_hip_error()); defined beside that function.
+void record_hip_error(int hip_error);
+
 struct FwdParams {
   const uint16_t* q;
   const uint16_t* k;

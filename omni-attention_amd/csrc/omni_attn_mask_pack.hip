@@ -18,6 +18,12 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+namespace omni_attn {
+// Keeps the hipError_t behind an OMNI_ATTN_ERR_LAUNCH for omni_attn_last_hip_error() (defined
+// beside that function).
+void record_hip_error(int hip_error);
+}  // namespace omni_attn
+
 namespace {
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
@@ -57,17 +63,24 @@ extern "C" int omni_attn_pack_partial_masks_gfx950(const uint8_t* partial_masks,
     return OMNI_ATTN_ERR_MISALIGNED;
   const size_t n_words = size_t(num_partial) * QB * (KB / 32);
   int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess ||
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e == hipSuccess && cus <= 0) e = hipErrorInvalidDevice;
+  if (e != hipSuccess) {
+    omni_attn::record_hip_error(int(e));
     return OMNI_ATTN_ERR_LAUNCH;
+  }
   const size_t want = (n_words + 255) / 256;
   const size_t cap = size_t(cus) * 16;  // grid-stride beyond a few workgroups per compute unit
   const unsigned grid = unsigned(want < cap ? want : cap);
   const u32x4_t* src = reinterpret_cast<const u32x4_t*>(partial_masks);
   size_t n = n_words;
   void* args[] = {&src, &partial_bits, &n};
-  if (hipLaunchKernel(reinterpret_cast<const void*>(pack_mask_kernel), dim3(grid), dim3(256), args, 0,
-                      static_cast<hipStream_t>(stream)) != hipSuccess)
+  e = hipLaunchKernel(reinterpret_cast<const void*>(pack_mask_kernel), dim3(grid), dim3(256), args, 0,
+                      static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) {
+    omni_attn::record_hip_error(int(e));
     return OMNI_ATTN_ERR_LAUNCH;
+  }
   return OMNI_ATTN_OK;
 }

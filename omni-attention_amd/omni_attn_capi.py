@@ -27,8 +27,6 @@ EXPORTED_SYMBOLS = (
     "omni_attn_bwd_noalloc_gfx950",
     "omni_attn_bwd_noalloc_max_rows",
     "omni_attn_mfma_peak_probe_gfx950",
-    "omni_attn_mfma_mix_probe_gfx950",
-    "omni_attn_issue_probe_gfx950",
     "omni_attn_status_string",
     "omni_attn_last_hip_error",
     "omni_attn_abi_version",
@@ -59,13 +57,9 @@ def load_library() -> ctypes.CDLL:
         lib.omni_attn_bwd_noalloc_gfx950.argtypes = [vp] * 15 + [i32] * 11 + [ctypes.c_float, vp]
         lib.omni_attn_mfma_peak_probe_gfx950.restype = i32
         lib.omni_attn_mfma_peak_probe_gfx950.argtypes = [i32, i32, vp, ctypes.POINTER(ctypes.c_double), vp]
-        lib.omni_attn_mfma_mix_probe_gfx950.restype = i32
-        lib.omni_attn_mfma_mix_probe_gfx950.argtypes = [i32, i32, vp, vp, ctypes.POINTER(ctypes.c_double), vp]
         lib.omni_attn_status_string.restype = ctypes.c_char_p
         lib.omni_attn_status_string.argtypes = [i32]
         lib.omni_attn_last_hip_error.restype = i32
-        lib.omni_attn_issue_probe_gfx950.restype = i32
-        lib.omni_attn_issue_probe_gfx950.argtypes = [i32, i32, i32, i32, vp, vp]
         lib.omni_attn_abi_version.restype = i32
         _lib = lib
     return _lib
@@ -85,41 +79,6 @@ def mfma_peak_probe(dtype: int, iters: int, sink: torch.Tensor, stream: Optional
     if rc != 0:
         raise RuntimeError("omni_attn_mfma_peak_probe_gfx950: %s (status %d)" % (status_string(rc), rc))
     return flops.value
-
-
-def mfma_mix_probe(mix: int, iters: int, sink: torch.Tensor, ticks: Optional[torch.Tensor] = None,
-                   stream: Optional[int] = None) -> float:
-    """Enqueue the matrix-instruction loop with LDS operand reads (mix bit 1) and / or softmax vector
-    work (mix bit 2); returns the flop count of the launch.  `ticks`: two int64 on the GPU that
-    receive one wave's shader cycles and 100 MHz ticks."""
-    flops = ctypes.c_double(0.0)
-    if ticks is not None and not (ticks.is_cuda and ticks.dtype == torch.int64 and ticks.numel() >= 2
-                                  and ticks.is_contiguous()):
-        raise RuntimeError("ticks must be a contiguous int64 GPU tensor with two elements")
-    if stream is None:
-        stream = torch.cuda.current_stream(sink.device).cuda_stream
-    with torch.cuda.device(sink.device):
-        rc = load_library().omni_attn_mfma_mix_probe_gfx950(mix, iters, sink.data_ptr(), _ptr(ticks),
-                                                            ctypes.byref(flops), stream)
-    if rc != 0:
-        raise RuntimeError("omni_attn_mfma_mix_probe_gfx950: %s (status %d)" % (status_string(rc), rc))
-    return flops.value
-
-
-def issue_probe(n_plain: int, n_exp: int, waves_per_simd: int, iters: int, ticks: torch.Tensor,
-                stream: Optional[int] = None) -> None:
-    """Enqueue the issue probe: one workgroup, `waves_per_simd` waves per SIMD, groups of one matrix
-    instruction + `n_plain` v_fma_f32 + `n_exp` v_exp_f32.  `ticks`: at least 17 int64 on the GPU;
-    wave w's loop started at ticks[2w] and ended at ticks[2w + 1] (shader cycles)."""
-    if not (ticks.is_cuda and ticks.dtype == torch.int64 and ticks.numel() >= 17 and ticks.is_contiguous()):
-        raise RuntimeError("ticks must be a contiguous int64 GPU tensor with at least 17 elements")
-    if stream is None:
-        stream = torch.cuda.current_stream(ticks.device).cuda_stream
-    with torch.cuda.device(ticks.device):
-        rc = load_library().omni_attn_issue_probe_gfx950(n_plain, n_exp, waves_per_simd, iters, ticks.data_ptr(),
-                                                         stream)
-    if rc != 0:
-        raise RuntimeError("omni_attn_issue_probe_gfx950: %s (status %d)" % (status_string(rc), rc))
 
 
 def _ptr(t: Optional[torch.Tensor]) -> int:

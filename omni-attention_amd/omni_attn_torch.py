@@ -18,7 +18,7 @@ import importlib
 import math
 import os
 import sys
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from enum import IntEnum
 from typing import List, Optional, Sequence, Tuple, Union
 
@@ -66,6 +66,16 @@ class OmniBlockMask:
     partial_block_mask_indices: Optional[Tensor] = None
     partial_block_masks: Optional[Tensor] = None
     partial_block_bits: Optional[Tensor] = None
+    # cache of has_partial_slots(); travels with to()
+    _any_partial_slot: Optional[bool] = field(default=None, repr=False, compare=False)
+
+    def has_partial_slots(self) -> bool:
+        """Does any slot carry the type PARTIAL?  Answered once per mask (one reduction, and on a GPU
+        one read-back) and remembered: the wrappers that need the answer on every call
+        (omni_attn_torch.py:763-765, :1067-1069) then cost no device synchronisation."""
+        if self._any_partial_slot is None:
+            self._any_partial_slot = bool((self.block_mask_types == int(BlockMaskType.PARTIAL)).any())
+        return self._any_partial_slot
 
     def pack_partial_masks(self) -> "OmniBlockMask":
         """Pack the PARTIAL tiles once (on the GPU, by the extension's pre-pass kernel) for a mask
@@ -140,7 +150,8 @@ class OmniBlockMask:
         return OmniBlockMask(
             mv(self.kv_num_blocks), mv(self.kv_indices), mv(self.block_mask_types),
             self.q_len, self.kv_len, self.Q_BLOCK_SIZE, self.KV_BLOCK_SIZE,
-            mv(self.partial_block_mask_indices), mv(self.partial_block_masks), mv(self.partial_block_bits))
+            mv(self.partial_block_mask_indices), mv(self.partial_block_masks), mv(self.partial_block_bits),
+            self._any_partial_slot)
 
     def to_dense_mask(self, partial_fallback: str = "causal") -> Tensor:
         """Dense bool mask [B, H, q_len, kv_len], True = attend.
@@ -588,7 +599,7 @@ def _omni_attention(op_name: str, query: Tensor, key: Tensor, value: Tensor,
                    and block_mask.partial_block_masks is not None)
     if partial_needs_partial_types:
         # the simple / cp_async / prefetch wrappers also require a PARTIAL slot to exist
-        has_partial = has_partial and bool((block_mask_types == BlockMaskType.PARTIAL).any())
+        has_partial = has_partial and block_mask.has_partial_slots()
     if has_partial:
         partial_idx = block_mask.partial_block_mask_indices.to(device=dev, dtype=torch.int32).contiguous()
         partial_masks = block_mask.partial_block_masks.to(device=dev, dtype=torch.bool).contiguous()

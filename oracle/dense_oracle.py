@@ -87,6 +87,40 @@ def attention_dense_grads_closed_form(q, k, v, mask, dout):
     return torch.matmul(ds, kf) * scale, torch.matmul(ds.transpose(-1, -2), qf) * scale, dv
 
 
+def attention_dense_grads_chunked(q, k, v, mask, dout, row_chunk: int = 2048, softcap: float = 0.0):
+    """The closed form of attention_dense_grads_closed_form worked over blocks of query rows, so
+    that one [S, S] slab at S = 16384 needs a few hundred MB instead of several GB (q, k, v, dout:
+    [S, D]; mask: [S, S] bool).  With softcap > 0 the score gradient carries the derivative of
+    softcap * tanh(x / softcap), 1 - tanh^2.  Pinned against autograd in tests/test_oracle_pinning.py."""
+    qf, kf, vf, do = q.float(), k.float(), v.float(), dout.float()
+    S, D = qf.shape
+    scale = 1.0 / math.sqrt(D)
+    dq = torch.zeros_like(qf)
+    dk = torch.zeros_like(kf)
+    dv = torch.zeros_like(vf)
+    for r0 in range(0, S, row_chunk):
+        r1 = min(S, r0 + row_chunk)
+        m = mask[r0:r1]
+        x = torch.matmul(qf[r0:r1], kf.t()) * scale
+        dfac = None
+        if softcap > 0:
+            t = torch.tanh(x / softcap)
+            x = t * softcap
+            dfac = 1.0 - t * t
+        any_row = m.any(-1, keepdim=True)
+        x = torch.where(any_row, x.masked_fill(~m, float("-inf")), torch.zeros_like(x))
+        p = torch.where(any_row, torch.softmax(x, dim=-1), torch.zeros_like(x))
+        o = torch.matmul(p, vf)
+        delta = (do[r0:r1] * o).sum(-1, keepdim=True)
+        dv += torch.matmul(p.t(), do[r0:r1])
+        ds = p * (torch.matmul(do[r0:r1], vf.t()) - delta)
+        if dfac is not None:
+            ds = ds * dfac
+        dq[r0:r1] = torch.matmul(ds, kf) * scale
+        dk += torch.matmul(ds.t(), qf[r0:r1]) * scale
+    return dq, dk, dv
+
+
 def prefix_mask(prefix_len: torch.Tensor, kv_len: int) -> torch.Tensor:
     """allow[..., i, j] = j < prefix_len[..., i]."""
     j = torch.arange(kv_len, device=prefix_len.device)

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(omni_attn_capi.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert omni_attn_capi.load_library().omni_attn_abi_version() == 3
+    assert omni_attn_capi.load_library().omni_attn_abi_version() == 4
 
 
 def test_argument_validation_codes():
@@ -60,7 +60,7 @@ def test_python_module_surface():
                  "omni_attn_preftech_kernel", "omni_attn_preftech",
                  "omni_attn_mma_stages_split_q_shared_kv_swizzle", "omni_attn_forward"):
         assert callable(getattr(omni_attn, name)), name
-    assert omni_attn.abi_version() == 3
+    assert omni_attn.abi_version() == 4
     assert os.path.dirname(omni_attn.__file__) == PKG
 
 

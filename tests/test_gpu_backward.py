@@ -14,14 +14,16 @@ import torch
 import omni_attn_capi
 from baseline_configs import make_workload
 from helpers import random_block_metadata
-from oracle.dense_oracle import attention_dense_fp32, attention_dense_grads, dense_mask_from_blocks, prefix_mask
+from oracle.dense_oracle import (attention_dense_fp32, attention_dense_grads, attention_dense_grads_chunked,
+                                 dense_mask_from_blocks, prefix_mask)
 
 pytestmark = pytest.mark.gpu
 
 TOL_GRAD = {torch.float16: 4e-3, torch.bfloat16: 3e-2}
 
 
-def run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, seqlen, pidx=None, pm=None, device="cuda:0", packed=False):
+def run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, seqlen, pidx=None, pm=None, device="cuda:0", packed=False,
+                softcap=0.0):
     dev = lambda t: None if t is None else t.to(device).contiguous()
     qd, kd, vd, dod = dev(q), dev(k), dev(v), dev(dout)
     nbd, idxd, tysd, pidxd, pmd = dev(nb), dev(idx), dev(tys), dev(pidx), dev(pm)
@@ -29,12 +31,13 @@ def run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, seqlen, pidx=None, pm=None,
     o = torch.full_like(qd, float("nan"))
     lse = torch.full(qd.shape[:3], float("nan"), dtype=torch.float32, device=device)
     if bits is not None:
-        omni_attn_capi.fwd(qd, kd, vd, o, lse, nbd, idxd, tysd, QB, KB, seqlen, pidxd, None, partial_bits=bits)
+        omni_attn_capi.fwd(qd, kd, vd, o, lse, nbd, idxd, tysd, QB, KB, seqlen, pidxd, None, partial_bits=bits,
+                           softcap=softcap)
     else:
-        omni_attn_capi.fwd(qd, kd, vd, o, lse, nbd, idxd, tysd, QB, KB, seqlen, pidxd, pmd)
+        omni_attn_capi.fwd(qd, kd, vd, o, lse, nbd, idxd, tysd, QB, KB, seqlen, pidxd, pmd, softcap=softcap)
     dq, dk, dv = (torch.full_like(qd, float("nan")) for _ in range(3))
     omni_attn_capi.bwd(qd, kd, vd, o, dod, lse, dq, dk, dv, nbd, idxd, tysd, QB, KB, seqlen, pidxd,
-                       None if bits is not None else pmd, bits)
+                       None if bits is not None else pmd, bits, softcap=softcap)
     torch.cuda.synchronize()
     return dq, dk, dv, o, lse
 
@@ -74,21 +77,47 @@ def test_c3_partial_shrunk_backward(packed, gpu_device):
     check_grads(got[:3], ref, w.dtype, "c3 shrunk")
 
 
+@pytest.mark.parametrize("softcap", [0.0, 2.0, 50.0], ids=["nocap", "cap2", "cap50"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
 @pytest.mark.parametrize("D", [32, 64, 128])
 @pytest.mark.parametrize("QB,KB", [(128, 128), (128, 64), (64, 128), (64, 64)])
-def test_random_metadata_backward(dtype, D, QB, KB, gpu_device):
+def test_random_metadata_backward(dtype, D, QB, KB, softcap, gpu_device):
+    """Every instance of both backward kernels, plain and soft-capped (byte tiles, every slot kind,
+    a sequence that ends inside a block)."""
     gen = torch.Generator().manual_seed(7000 + 10 * D + QB + KB // 64)
     B, H, S = 2, 2, 512
     q, k, v, dout = (torch.randn(B, H, S, D, generator=gen).to(dtype) for _ in range(4))
     nb, idx, tys, pidx, pm = random_block_metadata(gen, B, H, S // QB, S // KB, QB, KB, shuffle=True)
     for seqlen in (S, S - 45):
-        got = run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, seqlen, pidx, pm, device=gpu_device)
+        got = run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, seqlen, pidx, pm, device=gpu_device, softcap=softcap)
         dense = dense_mask_from_blocks(nb, idx, tys, QB, KB, S, S, pidx, pm, seqlen_orig=seqlen)
-        ref = attention_dense_grads(q, k, v, dense, dout)
-        check_grads(got[:3], ref, dtype, f"random metadata seqlen={seqlen}")
+        ref = attention_dense_grads(q, k, v, dense, dout, softcap=softcap)
+        check_grads(got[:3], ref, dtype, f"random metadata seqlen={seqlen} softcap={softcap}")
         for t in got[:3]:
             assert (t[:, :, seqlen:] == 0).all(), "rows beyond the sequence must get zero gradients"
+
+
+def test_padding_rows_are_never_read(gpu_device):
+    """Rows at or beyond seqlen_orig of q, k, v and dO may hold anything (here NaN): the outputs
+    are the same bits as with zeros there, finite everywhere and zero on the padding."""
+    gen = torch.Generator().manual_seed(108)
+    B, H, S, seqlen = 1, 3, 384, 300
+    for dtype, D, QB, KB in ((torch.bfloat16, 128, 128, 128), (torch.float16, 64, 128, 64), (torch.bfloat16, 32, 64, 64)):
+        q, k, v, dout = (torch.randn(B, H, S, D, generator=gen).to(dtype) for _ in range(4))
+        nb, idx, tys, pidx, pm = random_block_metadata(gen, B, H, S // QB, S // KB, QB, KB, shuffle=True)
+        clean = []
+        for t in (q, k, v, dout):
+            t[:, :, seqlen:] = 0
+            clean.append(t.clone())
+        ref = run_fwd_bwd(*clean, nb, idx, tys, QB, KB, seqlen, pidx, pm, device=gpu_device)
+        for t in (q, k, v, dout):
+            t[:, :, seqlen:] = float("nan")
+        got = run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, seqlen, pidx, pm, device=gpu_device)
+        for name, a, b in zip(("dQ", "dK", "dV", "O", "LSE"), got, ref):
+            assert name == "LSE" or torch.isfinite(a).all(), f"non-finite {name}"
+            assert not torch.isnan(a).any() and torch.equal(a, b), f"{name} depends on the padding rows"
+        for t in got[:4]:
+            assert (t[:, :, seqlen:] == 0).all()
 
 
 def test_sequences_of_length_zero_and_one(gpu_device):
@@ -181,6 +210,35 @@ def test_c2_full_size_backward_on_sampled_slabs(gpu_device):
         mask = prefix_mask(w.prefix_len[b], S)
         ref = attention_dense_grads(w.q[b, h], w.k[b, h], w.v[b, h], mask, dout[b, h])
         check_grads([t[b, h] for t in cpu], ref, w.dtype, f"c2 slab ({b},{h})")
+
+
+FULL_SIZE_SLABS = {
+    "c3_partial": [(0, 0), (0, 5), (0, 10), (0, 15)],
+    "c4_long": [(0, 0), (0, 9), (0, 18), (0, 27)],
+    "c5_batched": [(b, (5 * b + 1) % 16) for b in range(8)],  # every batch layout
+}
+
+
+@pytest.mark.parametrize("name,packed", [("c3_partial", False), ("c3_partial", True), ("c4_long", False),
+                                         ("c5_batched", False)],
+                         ids=["c3_partial-bytes", "c3_partial-bits", "c4_long", "c5_batched"])
+def test_config_full_size_backward_on_sampled_slabs(name, packed, gpu_device):
+    """BASELINE configurations 3, 4 and 5 at full size: the whole backward runs on the GPU, sampled
+    (batch, head) slabs are compared with the closed-form fp32 gradients of the dense oracle."""
+    w = make_workload(name, seed=0)
+    m = w.block_mask
+    B, H, S, D = w.q.shape
+    gen = torch.Generator().manual_seed(109)
+    dout = torch.randn(w.q.shape, generator=gen).to(w.dtype)
+    got = run_fwd_bwd(w.q, w.k, w.v, dout, m.kv_num_blocks, m.kv_indices, m.block_mask_types, m.Q_BLOCK_SIZE,
+                      m.KV_BLOCK_SIZE, S, m.partial_block_mask_indices, m.partial_block_masks,
+                      device=gpu_device, packed=packed)
+    for t in got[:3]:
+        assert torch.isfinite(t).all()
+    for b, h in FULL_SIZE_SLABS[name]:
+        mask = prefix_mask(w.prefix_len[b], S)
+        ref = attention_dense_grads_chunked(w.q[b, h], w.k[b, h], w.v[b, h], mask, dout[b, h])
+        check_grads([t[b, h] for t in got[:3]], ref, w.dtype, f"{name} slab ({b},{h})")
 
 
 def test_duplicate_and_clamped_block_indices_backward(gpu_device):

@@ -309,6 +309,53 @@ def test_wide_score_range_moves_the_reference_often(dtype, gain, gpu_device):
     assert rel_l <= TOL_LSE, f"gain {gain}: LSE relative error {rel_l:.3e}"
 
 
+def sparse_rows_bf16_case():
+    """B=2 H=9 S=1152 D=128 128/128 bf16, standard-normal operands, 80 % of the blocks left out
+    and shuffled lists: many rows attend one, two or a handful of keys, so outputs are single V
+    entries of magnitude 2 .. 4.7 instead of averages near 0."""
+    gen = torch.Generator().manual_seed(19073)
+    B, H, S, D, QB, KB = 2, 9, 1152, 128, 128, 128
+    q, k, v = (torch.randn(B, H, S, D, generator=gen).to(torch.bfloat16) for _ in range(3))
+    meta = random_block_metadata(gen, B, H, S // QB, S // KB, QB, KB, p_empty=0.8, shuffle=True)
+    return (q, k, v) + tuple(meta) + (QB, KB, S)
+
+
+def two_rounding_bound(q, k, v, dense, dtype):
+    """What the two roundings to the 16-bit type can cost an output element: the weights P are
+    rounded before the PV product while the row sum keeps the unrounded ones (relative error u
+    per weight: at most u * sum_j p_j |v_j| / l), and the result is rounded once more (u * |O|);
+    u = 2^-8 for bf16 (8 significant bits), 2^-11 for fp16."""
+    u = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    ref, _ = attention_dense_fp32(q, k, v, dense)
+    mean_abs, _ = attention_dense_fp32(q, k, v.float().abs(), dense)
+    return ref, u * (mean_abs + ref.abs()) + 1e-4
+
+
+def test_bf16_error_on_rows_with_few_keys_is_the_two_roundings(gpu_device):
+    """With bf16 the north-star bar of 1e-2 is an absolute one, and an output of magnitude 2 .. 4
+    already moves by up to 2^-7 = 0.0078 when it is rounded to bf16; rounding P before the PV
+    product (as the reference does, omni_attn_shared_kv.cu:450-453) adds up to 2^-8 * |V|.  On this
+    input the largest deviation is 0.0114 (row 634 of slab (0, 2): keys 949 and 964, weights 0.0745
+    and 0.9255, V = 0.516 and -2.781; the walk meets the small weight first, so the large one is
+    12.416 -> 12.4375 in bf16 against a row sum of 13.416: -2.53999, which rounds to -2.546875;
+    fp32 gives -2.535505).  Asserted: every element within the bound of the two roundings; the
+    plain bar wherever that bound is below it; LSE and empty rows as everywhere."""
+    q, k, v, nb, idx, tys, pidx, pm, QB, KB, S = sparse_rows_bf16_case()
+    o, lse = run_kernel(q, k, v, nb, idx, tys, QB, KB, S, pidx, pm, device=gpu_device)
+    dense = dense_mask_from_blocks(nb, idx, tys, QB, KB, S, S, pidx, pm, seqlen_orig=S)
+    ref, bound = two_rounding_bound(q, k, v, dense, torch.bfloat16)
+    _, rl = attention_dense_fp32(q, k, v, dense)
+    o32, l32 = o.float().cpu(), lse.float().cpu()
+    err = (o32 - ref).abs()
+    assert (err <= bound).all(), f"max excess over the rounding bound {(err - bound).max().item():.3e}"
+    inside = bound <= TOL_O[torch.bfloat16]
+    assert inside.float().mean().item() > 0.9 and err[inside].max().item() <= TOL_O[torch.bfloat16]
+    assert err.max().item() <= TOL_O[torch.bfloat16] + 2.0 ** -8 * v.float().abs().max().item()
+    empty = torch.isinf(rl) & (rl < 0)
+    assert torch.equal(torch.isinf(l32) & (l32 < 0), empty) and (o32[empty] == 0).all()
+    assert (l32[~empty] - rl[~empty]).abs().max().item() <= TOL_LSE
+
+
 def test_the_forward_can_be_captured_in_a_graph(gpu_device):
     """No entry point allocates or keeps state: a captured launch replays with new contents
     of the same buffers.  Replays are interleaved with eager work and synchronisations and

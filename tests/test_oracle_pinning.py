@@ -261,3 +261,130 @@ def test_gradient_oracle_one_allowed_key_per_row():
     assert dq.abs().max() < 1e-6 and dk.abs().max() < 1e-6
     expect = torch.zeros(S, D).index_add_(0, target, dout)
     assert torch.allclose(dv, expect, atol=1e-6)
+
+
+# ---- the soft-capped branch of the oracle -------------------------------------------------------
+# (transfusion_pytorch/transfusion.py:298-299 softclamp; :966-968: applied to the SCALED score,
+# before the mask).  None of the checks below evaluates softcap * tanh(x / softcap) with torch.
+
+def test_softcap_limits():
+    gen = torch.Generator().manual_seed(41)
+    S, D = 12, 8
+    q, k, v = (_rand(gen, S, D) for _ in range(3))
+    mask = torch.rand(S, S, generator=gen) < 0.5
+    mask[5] = False
+    # cap -> infinity: the plain oracle (tanh(x) = x - x^3/3 + ...: relative deviation (x / cap)^2 / 3)
+    o0, l0 = attention_dense_fp32(q, k, v, mask)
+    o1, l1 = attention_dense_fp32(q, k, v, mask, softcap=1e6)
+    live = ~torch.isinf(l0)
+    assert torch.allclose(o0, o1, atol=1e-6) and torch.allclose(l0[live], l1[live], atol=1e-6)
+    assert torch.equal(torch.isinf(l0), torch.isinf(l1)) and (o1[5] == 0).all()
+    # cap -> 0: every allowed score lies in [-cap, cap], so the weights are uniform up to
+    # exp(2 cap): mean of the allowed V rows, lse = log n +- cap
+    cap = 1e-3
+    o2, l2 = attention_dense_fp32(q, k, v, mask, softcap=cap)
+    for i in range(S):
+        n = int(mask[i].sum())
+        if n == 0:
+            assert (o2[i] == 0).all() and l2[i] == float("-inf")
+            continue
+        assert torch.allclose(o2[i], v[mask[i]].mean(0), atol=4 * cap * v.abs().max().item())
+        assert abs(l2[i].item() - math.log(n)) <= cap + 1e-6
+
+
+def test_softcap_two_key_row_by_hand():
+    """One query, two keys, worked with math.tanh / math.exp: the cap acts on q.k / sqrt(D)."""
+    q = torch.tensor([[1.5, -2.0, 0.5, 3.0]])
+    k = torch.tensor([[2.0, 1.0, -1.0, 4.0], [-3.0, 0.5, 2.0, -1.0]])
+    v = torch.tensor([[1.0, 10.0], [-2.0, 4.0]])
+    cap = 2.0
+    x = [sum(float(a) * float(b) for a, b in zip(q[0], k[j])) / 2.0 for j in range(2)]  # sqrt(4) = 2
+    assert x == [6.25, -3.75]
+    y = [cap * math.tanh(xi / cap) for xi in x]
+    z = [math.exp(yi) for yi in y]
+    expect_o = [(z[0] * float(v[0, d]) + z[1] * float(v[1, d])) / (z[0] + z[1]) for d in range(2)]
+    expect_l = math.log(z[0] + z[1])
+    qq = torch.cat([q, torch.zeros(1, 4)])          # two rows (the second attends nothing)
+    mask = torch.tensor([[True, True], [False, False]])
+    o, lse = attention_dense_fp32(qq, k, v, mask, softcap=cap)
+    assert abs(o[0, 0].item() - expect_o[0]) < 1e-6 and abs(o[0, 1].item() - expect_o[1]) < 1e-6
+    assert abs(lse[0].item() - expect_l) < 1e-6
+    # a cap applied to the raw product (12.5 and -7.5, saturated at +-2 as well, but
+    # by different amounts) or after the mask would give other numbers:
+    y_raw = [cap * math.tanh(2.0 * xi / cap) / 2.0 for xi in x]
+    assert abs(y_raw[0] - y[0]) > 0.5
+
+
+def test_softcap_acts_on_the_scaled_score():
+    """Zero-padding the head dimension to 4 D halves every scaled score and leaves q.k alone: with
+    the cap on the scaled score the result equals that of scores halved before the cap."""
+    gen = torch.Generator().manual_seed(42)
+    S, D = 10, 8
+    q, k, v = (_rand(gen, S, D) * 3 for _ in range(3))
+    causal = torch.tril(torch.ones(S, S, dtype=torch.bool))
+    pad = torch.zeros(S, 3 * D)
+    a, la = attention_dense_fp32(torch.cat([q, pad], -1), torch.cat([k, pad], -1), v, causal, softcap=1.5)
+    b, lb = attention_dense_fp32(q / 2.0, k, v, causal, softcap=1.5)
+    assert torch.allclose(a, b, atol=1e-6) and torch.allclose(la, lb, atol=1e-6)
+    c, _ = attention_dense_fp32(q, k, v, causal, softcap=1.5)
+    assert (a - c).abs().max() > 1e-2  # and the cap is not scale-invariant
+
+
+def test_softcap_per_element_loop_and_gradcheck():
+    from oracle.dense_oracle import (attention_dense_differentiable, attention_dense_grads,
+                                     attention_dense_grads_chunked)
+    gen = torch.Generator().manual_seed(43)
+    S, D, cap = 6, 4, 0.8
+    q, k, v = (_rand(gen, S, D) * 2 for _ in range(3))
+    mask = torch.rand(S, S, generator=gen) < 0.6
+    mask[2] = False
+    o, lse = attention_dense_fp32(q, k, v, mask, softcap=cap)
+    for i in range(S):
+        ws = {}
+        for j in range(S):
+            if mask[i, j]:
+                x = sum(float(q[i, d]) * float(k[j, d]) for d in range(D)) / math.sqrt(D)
+                ws[j] = math.exp(cap * math.tanh(x / cap))
+        if not ws:
+            assert (o[i] == 0).all() and lse[i] == float("-inf")
+            continue
+        tot = sum(ws.values())
+        for d in range(D):
+            assert abs(o[i, d].item() - sum(w * float(v[j, d]) for j, w in ws.items()) / tot) < 1e-5
+        assert abs(lse[i].item() - math.log(tot)) < 1e-5
+    q64, k64, v64 = (t.double().requires_grad_(True) for t in (q, k, v))
+    assert torch.autograd.gradcheck(lambda a, b, c: attention_dense_differentiable(a, b, c, mask, cap),
+                                    (q64, k64, v64), eps=1e-6, atol=1e-6)
+    # the row-blocked closed form (with the cap's derivative 1 - tanh^2) against autograd
+    dout = _rand(gen, S, D)
+    for sc in (0.0, cap):
+        auto = attention_dense_grads(q, k, v, mask, dout, softcap=sc)
+        for chunk in (4, 64):
+            form = attention_dense_grads_chunked(q, k, v, mask, dout, row_chunk=chunk, softcap=sc)
+            for a, b in zip(auto, form):
+                assert torch.allclose(a, b, atol=2e-6), (a - b).abs().max()
+
+
+# ---- what rounding P and O to bf16 costs (the limit of the absolute bar on sparse rows) ----------
+
+def test_bf16_two_rounding_model_on_a_two_key_row():
+    """The row the GPU test test_bf16_error_on_rows_with_few_keys_is_the_two_roundings quotes, by
+    hand: weights 1 : 12.416 (the walk meets the small one first, so the reference point of the
+    exponentials stays at it), V = 0.515625 and -2.78125.  fp32: -2.5355.  With the large weight
+    rounded to bf16 (12.4375) over the unrounded row sum: -2.53999, which bf16 rounds away from the
+    fp32 value to -2.546875: 0.0114 from the oracle, beyond the absolute bar of 1e-2, inside
+    2^-8 (sum p |v| / l + |O|)."""
+    p_small, p_large = 1.0, 1.0 / 0.08054216206073761
+    v_small, v_large = 0.515625, -2.78125
+    exact = (p_small * v_small + p_large * v_large) / (p_small + p_large)
+    assert abs(exact - (-2.535505)) < 1e-5
+    rounded_p = torch.tensor(p_large).to(torch.bfloat16).item()
+    assert rounded_p == 12.4375
+    kernel_fp32 = (p_small * v_small + rounded_p * v_large) / (p_small + p_large)
+    assert abs(kernel_fp32 - (-2.53999)) < 1e-5
+    out = torch.tensor(kernel_fp32).to(torch.bfloat16).item()
+    assert out == -2.546875
+    err = abs(out - exact)
+    assert 1e-2 < err < 1.2e-2
+    mean_abs = (p_small * abs(v_small) + p_large * abs(v_large)) / (p_small + p_large)
+    assert err <= 2.0 ** -8 * (mean_abs + abs(exact))
