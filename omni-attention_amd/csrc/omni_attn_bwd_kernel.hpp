@@ -13,7 +13,7 @@
 //
 // Two kernels, no atomics, bitwise reproducible:
 //   bwd_dq_kernel    one workgroup per query block; walks that block's list like the forward;
-//                    also writes -delta and the rows' exponent offsets (workspace, read by the
+//                    also writes -delta and the rows' score offsets (workspace, read by the
 //                    second kernel).
 //   bwd_dkdv_kernel  one workgroup per KV block; finds the (query block, slot) pairs that list
 //                    it by scanning the slab's metadata (a bitmap of the matches is built in
@@ -25,10 +25,15 @@
 // the same tile) and whose B operand is in registers, and the accumulator of the first product
 // of a step is the B operand of the second one, so P and dS never leave registers (the dK/dV
 // kernel hands P from one wave to its partner through LDS).
-// Tiles are loaded one step ahead (one barrier per step) and the fragments of a product are read
-// ahead of it; inside a step the order of the products and the vector work is pinned, the rest
-// is the compiler's schedule.  Workgroups are dealt to the XCDs by slab, so the workgroups that
-// run together on an XCD share their operands through its L2.
+// Tiles are loaded one step ahead (one barrier per step).  A step of 64 rows (or keys) is two
+// 32-wide halves and runs as one sequence of slots like an iteration of the forward: one MFMA,
+// the LDS fetch of an operand two or three slots ahead and a share of the vector work of the
+// half whose first products have just finished, with a scheduling fence after every slot -- the
+// exponentials of one half run under the products of the other inside one wave.  Offsets
+// (-LSE sqrt(D), -delta) and masks (-inf) go into the accumulators the products start from, so a
+// weight is one multiplication and one exp2 and an unmasked step carries no mask instruction.
+// Workgroups are dealt to the XCDs by slab, so the workgroups that run together on an XCD share
+// their operands through its L2.
 #pragma once
 
 #include "omni_attn_fwd_kernel.hpp"
@@ -106,6 +111,12 @@ __device__ __forceinline__ u32x4_t lds_tr_pair_at(uint32_t lo_addr, uint32_t hi_
   const u32x4_t a = {lo2[0], lo2[1], hi2[0], hi2[1]};
   return a;
 }
+// A transposed A fragment at (tile + lane part of its first half) ^ (column bits) + a constant:
+// the second half lies 8 tile rows further, where every swizzle differs by chunk bit 1 (32 bytes).
+template <int D>
+__device__ __forceinline__ u32x4_t lds_tr_frag(uint32_t lo_lane, uint32_t col_bits, uint32_t off) {
+  return lds_tr_pair_at((lo_lane ^ col_bits) + off, (lo_lane ^ (col_bits ^ 32u)) + off + 8u * D * 2u);
+}
 
 // One LDS layout serves both kinds of operand reads of a backward tile ([rows][D] 16-bit, the
 // 16-byte chunk index of a row XORed with a function of the row, period 16 rows):
@@ -147,12 +158,20 @@ __device__ __forceinline__ void bwd_load_tile(i32x4_t rsrc, int row0, uint32_t l
   constexpr int ROW_STRIDE = NT / CPR;
   if (TOTAL < NT && tid >= TOTAL) return;  // a small tile is loaded by the first waves only
   const int ld_row = tid / CPR, ld_pch = tid % CPR;
+  // The swizzle repeats every 16 rows and a thread's loads are ROW_STRIDE rows apart: one or two
+  // per-lane offsets serve all of them, the rest of the address is wave-uniform.
+  constexpr int PER = (NCH == 1 || ROW_STRIDE % 16 == 0) ? 1 : 2;
+  static_assert(NCH == 1 || (PER * ROW_STRIDE) % 16 == 0, "swizzle must repeat over a thread's loads");
+  uint32_t lane_off[PER];
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
+  for (int i = 0; i < PER; ++i) {
     const int row = ld_row + i * ROW_STRIDE;
-    const uint32_t off = uint32_t(row * D + (ld_pch ^ bwd_swizzle<D>(row)) * 8) * 2u;
-    buffer_to_lds_b128(rsrc, off, uint32_t(row0) * uint32_t(D * 2), lds_tile + uint32_t(w) * 1024u + uint32_t(i) * (NT * 16u));
+    lane_off[i] = uint32_t(row * D + (ld_pch ^ bwd_swizzle<D>(row)) * 8) * 2u - uint32_t(i * ROW_STRIDE * D * 2);
   }
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+    buffer_to_lds_b128(rsrc, lane_off[i % PER], uint32_t(row0 + i * ROW_STRIDE) * uint32_t(D * 2),
+                       lds_tile + uint32_t(w) * 1024u + uint32_t(i) * (NT * 16u));
 }
 
 // 32 mask bytes -> 32 bits (any non-zero byte = 1), byte i -> bit i.
@@ -203,12 +222,6 @@ __device__ __forceinline__ void bwd_store_rows(const f32x16_t (&acc)[D / 32], fl
   }
 }
 
-// Rows of a backward tile: 32 where a [32][D] tile still divides over the workgroup (two sets
-// of tiles then leave room for two workgroups per compute unit), else 64.
-template <int D, int NT>
-struct BwdRows {
-  static constexpr int value = (32 * (D / 8) % NT == 0) ? 32 : 64;
-};
 
 // One step of a backward walk.
 struct BwdStepInfo {
@@ -223,7 +236,8 @@ struct BwdStepInfo {
 template <int D, int QB>
 struct BwdDqTraits {
   static constexpr int kThreads = QB * 2;
-  static constexpr int kStep = BwdRows<D, kThreads>::value;
+  // keys per step: two 32-key halves whose products and vector work overlap inside a wave
+  static constexpr int kStep = 64;
   static constexpr int kTileElems = kStep * D;
   // two sets of two tiles (K, V), or the output staging
   static constexpr size_t kLdsBytes = (4 * kTileElems > QB * D ? 4 * kTileElems : QB * D) * sizeof(uint16_t);
@@ -271,7 +285,7 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
   const bool has_partial = p.partial_idx != nullptr && (p.partial_masks != nullptr || p.partial_bits != nullptr);
 
   // Block metadata in registers, as in the forward: lane i holds block 64 * chunk + i of the list.
-  int32_t mv_kvb = 0, mv_mode = kMasked, mv_pid = -1;
+  int32_t mv_kvb = 0, mv_info = kMasked;  // info: effective mode in the low two bits, tile index above
   auto load_chunk = [&](int chunk) {
     const int j = chunk * 64 + lane;
     const size_t o = meta_off + size_t(j < p.max_blocks ? j : 0);
@@ -279,8 +293,8 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
     const int32_t ty = p.types[o];
     const int32_t pid = has_partial ? p.partial_idx[o] : -1;
     mv_kvb = raw < 0 ? 0 : (raw >= p.Tk ? p.Tk - 1 : raw);
-    mv_mode = bwd_slot_mode(ty, pid, has_partial, p.num_partial);
-    mv_pid = pid;
+    const int32_t mode = bwd_slot_mode(ty, pid, has_partial, p.num_partial);
+    mv_info = (mode == kPartial ? pid << 2 : 0) | mode;
   };
   load_chunk(0);
   int nb = load_uniform(p.kv_num_blocks + meta_row);
@@ -366,8 +380,8 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
       if ((gj & 63) == 0 && gj > 0) load_chunk(gj >> 6);
       const int ln = gj & 63;
       const int kvb = __builtin_amdgcn_readlane(mv_kvb, ln);
-      const int mode = __builtin_amdgcn_readlane(mv_mode, ln);
-      const int pid = __builtin_amdgcn_readlane(mv_pid, ln);
+      const int info = __builtin_amdgcn_readlane(mv_info, ln);
+      const int mode = info & 3, pid = info >> 2;
       ++gj;
       const int row0 = kvb * KB;
       if (mode == kMasked || row0 >= p.seqlen || (mode == kCausal && row0 > q_last)) continue;
@@ -387,83 +401,104 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
     bwd_load_tile<D, NT, STEP>(rV, st.row0, base + TILE * 2u, tid, w);
   };
   const uint32_t row_lane = bwd_row_lane<D>(g, c);
-  const uint32_t tr_lo = bwd_tr_lane<D>(g, c, 0), tr_hi = bwd_tr_lane<D>(g, c, 1);
-  constexpr int PF = KS < 3 ? KS : 3;  // k-steps whose fragments are read ahead of their products
-
-  // One step: S^T = K.Q^T and dP^T = V.dO^T (lane = query row, registers = keys), then
-  // dS^T = P^T (dP^T - delta) packed to 16 bits in the order the next product reads it, then
-  // dQ^T += K^T.dS^T.
-  auto compute = [&](int set, const uint32_t (&kw)[NTL], bool all_allowed) {
+  const uint32_t tr_lo = bwd_tr_lane<D>(g, c, 0);
+  // One step, as one sequence of slots -- first the products S^T = K.Q^T and dP^T = V.dO^T of the
+  // 32-key halves (lane = query row, registers = keys; the two products of a k-step alternate),
+  // then the products dQ^T += K^T.dS^T of the halves -- each slot one MFMA, the LDS fetch of the
+  // operand three slots ahead and a share of the vector work of the half whose first products
+  // have just finished: dS^T = P^T (dP^T - delta), packed to 16 bits in the order the last
+  // product reads it, is computed for half u under the first products of half u + 1 (or under the
+  // last products of half 0).  The accumulator of S^T starts at the row's offset -LSE * sqrt(D) --
+  // at -inf where the step's mask forbids the pair (`masked`, wave-uniform) -- so that a weight is
+  // exp2(score * sl2); that of dP^T starts at -delta.  A soft-capped score is not linear in the
+  // product: there S^T starts at zero and offset and mask are applied to the weights.
+  constexpr int NSUB = NTL;
+  constexpr int NTR = 2 * DT;                    // last products of a half
+  constexpr int NS = NSUB * (2 * KS + NTR);      // slots of a step
+  constexpr int PF = D == 128 ? 2 : 3;           // operand fetch distance in slots (registers are tight at 128)
+  const float row_off = CAP ? lse2 : (row_live ? -lse * SqrtOf<D>::value : -INFINITY);
+  const float neg_delta = -delta;
+  auto compute = [&](int set, const uint32_t (&kw)[NTL], bool masked) {
     const uint32_t base = lds_tiles + uint32_t(set) * (2u * TILE * 2u);
-    const uint32_t aK = base + row_lane, aV = aK + TILE * 2u, tK0 = base + tr_lo, tK1 = base + tr_hi;
-    f32x16_t st[NTL], dp[NTL];
-    __builtin_amdgcn_s_setprio(1);  // products first: the other wave of the SIMD fills the gaps
-    static_for<NTL>([&](auto tc) {
-      constexpr int t = decltype(tc)::value;
-      constexpr uint32_t trow = uint32_t(t) * 32u * D * 2u;
-      u32x4_t fa[KS], fb[KS];
-      static_for<PF>([&](auto sc) {
-        constexpr int s = decltype(sc)::value;
-        fa[s] = lds_b128_at((aK ^ uint32_t(32 * s)) + trow);
-        fb[s] = lds_b128_at((aV ^ uint32_t(32 * s)) + trow);
-      });
-      static_for<KS>([&](auto sc) {
-        constexpr int s = decltype(sc)::value;
-        if constexpr (s + PF < KS) {
-          fa[s + PF] = lds_b128_at((aK ^ uint32_t(32 * (s + PF))) + trow);
-          fb[s + PF] = lds_b128_at((aV ^ uint32_t(32 * (s + PF))) + trow);
-        }
-        st[t] = mfma_32x32x16<BF16>(fa[s], qf[s], s == 0 ? zero16 : st[t]);
-        dp[t] = mfma_32x32x16<BF16>(fb[s], dof[s], s == 0 ? zero16 : dp[t]);
-        __builtin_amdgcn_sched_barrier(0);
-      });
-    });
-    constexpr int NTS = STEP / 16;
-    u32x4_t ft[NTS][DT];  // fragments of the second product, read one 16-key group ahead
-    static_for<DT>([&](auto dc) {
-      constexpr int dt = decltype(dc)::value;
-      ft[0][dt] = lds_tr_pair_at(tK0 ^ uint32_t(64 * dt), tK1 ^ uint32_t(64 * dt));
-    });
-    __builtin_amdgcn_s_setprio(0);
-    __builtin_amdgcn_sched_barrier(0);
-    u32x4_t dsb[NTL][2];
-    auto weights = [&](auto masked_c) {
-      constexpr bool MASKED = decltype(masked_c)::value;
-      static_for<8 * NTL>([&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        constexpr int t = i / 8, r = 2 * (i % 8);
-        constexpr int kl0 = 8 * (r >> 2) + (r & 3), kl1 = 8 * ((r + 1) >> 2) + ((r + 1) & 3);
-        float p0, p1, f0, f1;
-        bwd_weight<CAP>(st[t][r], lse2, p, p0, f0);
-        bwd_weight<CAP>(st[t][r + 1], lse2, p, p1, f1);
-        if constexpr (MASKED) {
-          p0 = ((kw[t] >> kl0) & 1u) ? p0 : 0.f;
-          p1 = ((kw[t] >> kl1) & 1u) ? p1 : 0.f;
-        }
-        const float d0 = p0 * (dp[t][r] - delta) * f0;
-        const float d1 = p1 * (dp[t][r + 1] - delta) * f1;
-        dsb[t][r >> 3][(r & 7) >> 1] = pack2<BF16>(d0, d1);
-      });
-    };
-    if (all_allowed) {  // (wave-uniform) a FULL step inside the sequence needs no mask
-      weights(std::integral_constant<bool, false>{});
-    } else {
-      weights(std::integral_constant<bool, true>{});
-    }
-    __builtin_amdgcn_s_setprio(1);
-    static_for<NTS>([&](auto tsc) {
-      constexpr int ts = decltype(tsc)::value;
-      if constexpr (ts + 1 < NTS) {
-        static_for<DT>([&](auto dc) {
-          constexpr int dt = decltype(dc)::value;
-          ft[ts + 1][dt] = lds_tr_pair_at((tK0 ^ uint32_t(64 * dt)) + uint32_t(ts + 1) * 16u * D * 2u,
-                                          (tK1 ^ uint32_t(64 * dt)) + uint32_t(ts + 1) * 16u * D * 2u);
-        });
+    const uint32_t aK = base + row_lane, aV = aK + TILE * 2u, tK0 = base + tr_lo;
+    f32x16_t st[NSUB], dp[NSUB];
+    u32x4_t dsb[NSUB][2];
+    auto operand = [&](auto nc) {
+      constexpr int n = decltype(nc)::value;
+      if constexpr (n < NSUB * 2 * KS) {
+        constexpr int u = n / (2 * KS), s = (n % (2 * KS)) / 2, which = n % 2;
+        return lds_b128_at(((which ? aV : aK) ^ uint32_t(32 * s)) + uint32_t(u) * (32u * D * 2u));
+      } else {
+        constexpr int m = n - NSUB * 2 * KS, u = m / NTR, ts = (m % NTR) / DT, dt = m % DT;
+        constexpr uint32_t off = uint32_t(2 * u + ts) * (16u * D * 2u);
+        return lds_tr_frag<D>(tK0, uint32_t(64 * dt), off);
       }
-      static_for<DT>([&](auto dc) {
-        constexpr int dt = decltype(dc)::value;
-        dq[dt] = mfma_32x32x16<BF16>(ft[ts][dt], dsb[ts >> 1][ts & 1], dq[dt]);
-      });
+    };
+    auto keep_bits = [&](auto uc, auto rc) {  // 0 or ~0 for register r of half u
+      constexpr int u = decltype(uc)::value, r = decltype(rc)::value;
+      return uint32_t(__builtin_amdgcn_sbfe(int(kw[u]), 8 * (r >> 2) + (r & 3), 1));
+    };
+    // the score gradients of registers r, r + 1 of half u
+    auto grads = [&](auto uc, auto rc) {
+      constexpr int u = decltype(uc)::value, r = decltype(rc)::value;
+      float w0, w1, f0 = 1.f, f1 = 1.f;
+      if constexpr (CAP) {
+        bwd_weight<true>(st[u][r], row_off, p, w0, f0);
+        bwd_weight<true>(st[u][r + 1], row_off, p, w1, f1);
+        const uint32_t b0 = __builtin_bit_cast(uint32_t, w0) & keep_bits(uc, rc);
+        const uint32_t b1 = __builtin_bit_cast(uint32_t, w1) & keep_bits(uc, IntC<r + 1>{});
+        w0 = __builtin_bit_cast(float, b0) * f0;
+        w1 = __builtin_bit_cast(float, b1) * f1;
+      } else {
+        w0 = __builtin_amdgcn_exp2f(st[u][r] * p.sl2);
+        w1 = __builtin_amdgcn_exp2f(st[u][r + 1] * p.sl2);
+      }
+      dsb[u][r >> 3][(r & 7) >> 1] = pack2<BF16>(w0 * dp[u][r], w1 * dp[u][r + 1]);
+    };
+    u32x4_t opq[PF];
+    static_for<PF>([&](auto nc) { opq[decltype(nc)::value] = operand(nc); });
+    __builtin_amdgcn_s_setprio(1);  // products first: the other wave of the SIMD fills the gaps
+    static_for<NS>([&](auto nc) {
+      constexpr int n = decltype(nc)::value;
+      constexpr bool first = n < NSUB * 2 * KS;
+      constexpr int ch = first ? n / (2 * KS) : NSUB + (n - NSUB * 2 * KS) / NTR;  // chain of the slot
+      constexpr int sl = first ? n % (2 * KS) : (n - NSUB * 2 * KS) % NTR;          // slot inside it
+      constexpr int len = first ? 2 * KS : NTR;
+      if constexpr (first) {
+        constexpr int s = sl / 2;
+        if constexpr (sl == 0) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            st[ch][r] = CAP ? 0.f : row_off;
+            dp[ch][r] = neg_delta;
+          }
+          if constexpr (!CAP) {
+            if (masked) {
+              static_for<16>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                const uint32_t keep = keep_bits(IntC<ch>{}, rc);
+                const uint32_t bits = __builtin_bit_cast(uint32_t, float(st[ch][r]));
+                st[ch][r] = __builtin_bit_cast(float, (bits & keep) | (0xff800000u & ~keep));
+              });
+            }
+          }
+        }
+        if constexpr (sl % 2 == 0) {
+          st[ch] = mfma_32x32x16<BF16>(opq[n % PF], qf[s], st[ch]);
+        } else {
+          dp[ch] = mfma_32x32x16<BF16>(opq[n % PF], dof[s], dp[ch]);
+        }
+      } else {
+        constexpr int u = ch - NSUB, ts = sl / DT, dt = sl % DT;
+        dq[dt] = mfma_32x32x16<BF16>(opq[n % PF], dsb[u][ts], dq[dt]);
+      }
+      if constexpr (n + PF < NS) opq[n % PF] = operand(IntC<n + PF>{});
+      // the score gradients of half ch - 1 go beside the products of chain ch: 8 register pairs
+      // spread over the chain's slots
+      if constexpr (ch >= 1 && ch <= NSUB) {
+        constexpr int lo = sl * 8 / len, hi = (sl + 1) * 8 / len;
+        static_for<hi - lo>([&](auto ic) { grads(IntC<ch - 1>{}, IntC<2 * (lo + decltype(ic)::value)>{}); });
+      }
       __builtin_amdgcn_sched_barrier(0);
     });
     __builtin_amdgcn_s_setprio(0);
@@ -505,13 +540,27 @@ __global__ void __launch_bounds__(QB * 2, 2) bwd_dq_kernel(const BwdParams p) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this step's tiles (and mask words) have landed
     __syncthreads();                     // ... for every wave; and the other set is no longer read
     if (nxt.valid) issue_loads(nxt, set ^ 1);
-    compute(set, kw, cur.mode == kFull && cur.row0 + STEP <= p.seqlen);
+    compute(set, kw, !(cur.mode == kFull && cur.row0 + STEP <= p.seqlen));
     set ^= 1;
     cur = nxt;
   }
   __syncthreads();  // tiles are dead: the staging area overlaps them
   uint16_t* stage = lds16 + size_t(w) * 32 * D;
-  bwd_store_rows<BF16, D>(dq, p.scale, stage, p.dq + slab, q_wave_min, p.S, lane);
+  // (the lane number goes through an empty asm: the addresses of the epilogue are then computed
+  // here and not kept in registers across the walk, where every register counts)
+  int lane_out = lane;
+  asm volatile("" : "+v"(lane_out));
+  bwd_store_rows<BF16, D>(dq, p.scale, stage, p.dq + slab, q_wave_min, p.S, lane_out);
+}
+
+// First step of STEP query rows of query block qb that can contribute to KV block kvb: a CAUSAL
+// step whose rows all lie above the block's first key contributes nothing (the dK/dV kernel starts
+// a block's walk there, and never stores score gradients for the steps before it).
+template <int QB, int KB, int STEP>
+__device__ __forceinline__ int bwd_first_step(int mode, int kvb, int qb) {
+  if (mode != kCausal) return 0;
+  const int below = kvb * KB - (qb * QB + STEP - 1);  // rows of the block before the first useful step
+  return below > 0 ? (below + STEP - 1) / STEP : 0;
 }
 
 template <int D, int KB>
@@ -735,11 +784,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
       g_first = false;
       // first step of the match that contributes: CAUSAL steps entirely above the diagonal and
       // steps beyond the sequence do not
-      int sub = 0;
-      if (mode == kCausal) {
-        const int below = kvb * KB - (g_qb * QB + STEP - 1);  // rows of the block before the first useful step
-        sub = below > 0 ? (below + STEP - 1) / STEP : 0;
-      }
+      const int sub = bwd_first_step<QB, KB, STEP>(mode, kvb, g_qb);
       const int q0 = g_qb * QB + sub * STEP;
       if (sub >= NSTEPS || q0 >= p.seqlen) continue;
       g_last.row0 = q0;
@@ -772,12 +817,12 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
       buffer_to_lds_b32(rNd, uint32_t(rtid) * 4u, uint32_t(st.row0) * 4u, lds_nd + uint32_t(set * STEP) * 4u);
   };
   const uint32_t row_lane = bwd_row_lane<D>(g, c);
-  const uint32_t tr_lo = bwd_tr_lane<D>(g, c, 0), tr_hi = bwd_tr_lane<D>(g, c, 1);
+  const uint32_t tr_lo = bwd_tr_lane<D>(g, c, 0);
 
   // Operand n of a step's slot sequence, from the tile read row-wise (first products: rows
   // 32 u + lane of the tile at k-step s) or transposed (second products: columns 32 dt .. +31
   // at rows 32 u + 16 ts .. +15).
-  auto operand = [&](auto nc, uint32_t a_rows, uint32_t a_tr0, uint32_t a_tr1) {
+  auto operand = [&](auto nc, uint32_t a_rows, uint32_t a_tr0) {
     constexpr int n = decltype(nc)::value;
     constexpr int ch = n / KS, s = n % KS;
     if constexpr (ch < NSUB) {
@@ -785,7 +830,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
     } else {
       constexpr int u = ch - NSUB, ts = s / DT, dt = s % DT;
       constexpr uint32_t off = uint32_t(2 * u + ts) * (16u * D * 2u);
-      return lds_tr_pair_at((a_tr0 ^ uint32_t(64 * dt)) + off, (a_tr1 ^ uint32_t(64 * dt)) + off);
+      return lds_tr_frag<D>(a_tr0, uint32_t(64 * dt), off);
     }
   };
 
@@ -796,7 +841,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
   // soft-capped score is not linear in the product: there the accumulator starts at zero, the
   // offsets are fetched when the weights are computed and the mask is applied to the weights.
   auto weight_step = [&](int set, int par, const uint32_t (&kw)[NSUB], bool masked) {
-    const uint32_t aQ = tile_at(set, 0) + row_lane, tD0 = tile_at(set, 1) + tr_lo, tD1 = tile_at(set, 1) + tr_hi;
+    const uint32_t aQ = tile_at(set, 0) + row_lane, tD0 = tile_at(set, 1) + tr_lo;
     // The row offsets of the workspace: registers 4 i .. +3 of a half are its query rows
     // 8 i + 4 g .. +3.
     auto row_offsets = [&](int u, int i4) {
@@ -843,7 +888,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
       }
     };
     u32x4_t opq[PF];
-    static_for<PF>([&](auto nc) { opq[decltype(nc)::value] = operand(nc, aQ, tD0, tD1); });
+    static_for<PF>([&](auto nc) { opq[decltype(nc)::value] = operand(nc, aQ, tD0); });
     if constexpr (PRIO) __builtin_amdgcn_s_setprio(1);
     static_for<NS>([&](auto nc) {
       constexpr int n = decltype(nc)::value;
@@ -876,7 +921,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
         constexpr int u = ch - NSUB, ts = s / DT, dt = s % DT;
         acc[dt] = mfma_32x32x16<BF16>(opq[n % PF], pb[u][ts], acc[dt]);
       }
-      if constexpr (n + PF < NS) opq[n % PF] = operand(IntC<n + PF>{}, aQ, tD0, tD1);
+      if constexpr (n + PF < NS) opq[n % PF] = operand(IntC<n + PF>{}, aQ, tD0);
       // the weights of half ch - 1 go beside the products of chain ch
       if constexpr (NSUB > 1 && ch >= 1 && ch <= NSUB) weights(IntC<ch - 1>{}, IntC<s>{});
       __builtin_amdgcn_sched_barrier(0);
@@ -892,7 +937,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
   // Gradient wave, one step: dP - delta = dO.V^T - delta (the accumulator starts at -delta),
   // dS = P (dP - delta) with the partner's P, dK^T += Q^T.dS.
   auto grad_step = [&](int set, int par) {
-    const uint32_t aD = tile_at(set, 1) + row_lane, tQ0 = tile_at(set, 0) + tr_lo, tQ1 = tile_at(set, 0) + tr_hi;
+    const uint32_t aD = tile_at(set, 1) + row_lane, tQ0 = tile_at(set, 0) + tr_lo;
     f32x16_t dp[NSUB];
     u32x4_t hand[NSUB][2], dsb[NSUB][2];
     static_for<4 * NSUB>([&](auto ic) {
@@ -913,7 +958,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
       });
     };
     u32x4_t opq[PF];
-    static_for<PF>([&](auto nc) { opq[decltype(nc)::value] = operand(nc, aD, tQ0, tQ1); });
+    static_for<PF>([&](auto nc) { opq[decltype(nc)::value] = operand(nc, aD, tQ0); });
     if constexpr (PRIO) __builtin_amdgcn_s_setprio(1);
     static_for<NS>([&](auto nc) {
       constexpr int n = decltype(nc)::value;
@@ -928,7 +973,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
         constexpr int u = ch - NSUB, ts = s / DT, dt = s % DT;
         acc[dt] = mfma_32x32x16<BF16>(opq[n % PF], dsb[u][ts], acc[dt]);
       }
-      if constexpr (n + PF < NS) opq[n % PF] = operand(IntC<n + PF>{}, aD, tQ0, tQ1);
+      if constexpr (n + PF < NS) opq[n % PF] = operand(IntC<n + PF>{}, aD, tQ0);
       if constexpr (NSUB > 1 && ch >= 1 && ch <= NSUB) score_grads(IntC<ch - 1>{}, IntC<s>{});
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (NSUB == 1 && n == KS - 1) {
@@ -1053,12 +1098,12 @@ int launch_bwd_cap(const BwdParams& p, hipStream_t stream) {
   const unsigned slabs_per_xcd = unsigned(p.n_slabs + p.n_xcd - 1) / unsigned(p.n_xcd);
   BwdParams params = p;
   void* args[] = {&params};
-  e = hipLaunchKernel(reinterpret_cast<const void*>(kq), dim3(unsigned(p.n_xcd) * slabs_per_xcd * unsigned(p.Tq)),
-                      dim3(TQ::kThreads), args, TQ::kLdsBytes, stream);
+  const size_t dkdv_lds = TK::lds_bytes(size_t(p.Tq) * size_t((p.max_blocks + 63) / 64));
+  const dim3 dkdv_grid(unsigned(p.n_xcd) * slabs_per_xcd * unsigned(p.Tk));
+  const dim3 dq_grid(unsigned(p.n_xcd) * slabs_per_xcd * unsigned(p.Tq));
+  e = hipLaunchKernel(reinterpret_cast<const void*>(kq), dq_grid, dim3(TQ::kThreads), args, TQ::kLdsBytes, stream);
   if (e != hipSuccess) return int(e);
-  e = hipLaunchKernel(reinterpret_cast<const void*>(kk), dim3(unsigned(p.n_xcd) * slabs_per_xcd * unsigned(p.Tk)),
-                      dim3(TK::kThreads), args,
-                      TK::lds_bytes(size_t(p.Tq) * size_t((p.max_blocks + 63) / 64)), stream);
+  e = hipLaunchKernel(reinterpret_cast<const void*>(kk), dkdv_grid, dim3(TK::kThreads), args, dkdv_lds, stream);
   return int(e);
 }
 
