@@ -51,7 +51,7 @@ RESOURCES_JSON = os.path.join(OBJ, "kernel_resources.json")
 # least this many waves per SIMD (kernels are matched by a substring of their mangled name).
 # The backward kernels keep scalar values in spare vector lanes here and there (SGPR spills, no
 # memory behind them): for them only scratch memory and spilled vector registers fail the build.
-MIN_WAVES_PER_SIMD = {"fwd_kernel": 2, "bwd_dq_kernel": 2}
+MIN_WAVES_PER_SIMD = {"fwd_kernel": 2, "bwd_dq_kernel": 2, "bwd_dkdv_kernel": 2}
 SGPR_SPILLS_ALLOWED = ("bwd_dq_kernel", "bwd_dkdv_kernel")
 NOT_GATED = ("fwd_generic_kernel",)
 

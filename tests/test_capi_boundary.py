@@ -114,6 +114,15 @@ def test_kernel_resources_of_the_built_library():
     build.check_resources(kernels)
     for name, r in fwd.items():
         assert r["scratch_bytes"] == 0 and r["vgprs"] <= 256 and r["waves_per_simd"] >= 2, (name, r)
+    # both backward kernels, plain and soft-capped, 24 instances each way: two waves per SIMD or more
+    for tag in ("bwd_dq_kernel", "bwd_dkdv_kernel"):
+        inst = {k: v for k, v in kernels.items() if tag in k}
+        assert len(inst) == 48
+        for name, r in inst.items():
+            assert r["scratch_bytes"] == 0 and r["waves_per_simd"] >= 2, (name, r)
+    low_bwd = {"k_bwd_dkdv_kernel_x": {"scratch_bytes": 0, "vgpr_spills": 0, "sgpr_spills": 0, "waves_per_simd": 1}}
+    with pytest.raises(RuntimeError, match="waves per SIMD"):
+        build.check_resources(low_bwd)
     bad = {"k_fwd_kernel_x": {"scratch_bytes": 16, "vgpr_spills": 4, "sgpr_spills": 0, "waves_per_simd": 2}}
     with pytest.raises(RuntimeError, match="scratch"):
         build.check_resources(bad)

@@ -277,14 +277,15 @@ def test_runtime_is_linear_in_listed_blocks(gpu_device):
     assert r["fit"]["ns_per_block"] > 0
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
 @pytest.mark.parametrize("gain", [4.0, 12.0])
-def test_wide_score_range_moves_the_reference_often(dtype, gain, gpu_device):
+def test_wide_score_range_moves_the_reference_often(dtype, gain, D, gpu_device):
     """Scores whose running maximum keeps jumping by far more than 2^6 (the kernel's
     lazy reference point has to move, and O and l have to be rescaled, on many steps),
     rows that stay without any allowed key for several steps, and very negative scores."""
     gen = torch.Generator().manual_seed(int(gain) * 7 + (dtype == torch.float16))
-    B, H, S, D, QB, KB = 1, 3, 1536, 128, 128, 128
+    B, H, S, QB, KB = 1, 3, 1536, 128, 128
     q = (torch.randn(B, H, S, D, generator=gen) * gain).to(dtype)
     k = torch.randn(B, H, S, D, generator=gen).to(dtype)
     v = torch.randn(B, H, S, D, generator=gen).to(dtype)
@@ -306,6 +307,7 @@ def test_wide_score_range_moves_the_reference_often(dtype, gain, gpu_device):
     assert torch.equal(torch.isinf(l32) & (l32 < 0), empty)
     assert (o32[empty] == 0).all()
     rel_l = ((l32[~empty] - wl[~empty]).abs() / wl[~empty].abs().clamp(min=1.0)).max().item()
+    print(f"wide range D={D} {dtype} gain {gain}: max(|dO| - ulp|O|) = {excess:.3e}, LSE relative error {rel_l:.3e}")
     assert rel_l <= TOL_LSE, f"gain {gain}: LSE relative error {rel_l:.3e}"
 
 
