@@ -139,6 +139,24 @@ def cpu_baseline(w, budget_s: float):
     }
 
 
+def visited_pairs(m) -> int:
+    """(query row, key) pairs the scalar-semantics kernel visits: all of a FULL or PARTIAL block, the
+    keys up to the row's own position of a CAUSAL one."""
+    import torch
+    QB, KB = m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE
+    nb = m.kv_num_blocks.cpu().long()
+    slot = torch.arange(m.kv_indices.shape[-1]).view(1, 1, 1, -1)
+    live = slot < nb.unsqueeze(-1)
+    ty = m.block_mask_types.cpu().long()
+    kv0 = m.kv_indices.cpu().long() * KB
+    q0 = (torch.arange(nb.shape[2]) * QB).view(1, 1, -1, 1)
+    rows = torch.arange(QB).view(1, 1, 1, 1, -1)
+    causal = ((q0.unsqueeze(-1) + rows) - kv0.unsqueeze(-1) + 1).clamp(min=0, max=KB).sum(-1)
+    per_slot = torch.where(ty == 1, causal, torch.full_like(causal, QB * KB))
+    per_slot = torch.where(live & (ty != 0), per_slot, torch.zeros_like(per_slot))
+    return int(per_slot.sum().item())
+
+
 def band_sweep(dev, steps, warmup):
     """Kernel time against the number of listed blocks at the fixed shape of c2_interleaved
     (B=2, H=32, S=4096, D=128, bf16, 128/128): banded masks, query block i lists the FULL
@@ -343,6 +361,9 @@ def main(argv=None):
     ap.add_argument("--backward", action="store_true",
                     help="time the backward (dQ kernel + dK/dV kernel) instead of the forward; effective "
                          "flops are 10*QB*KB*D per listed block (five products)")
+    ap.add_argument("--generic-kernel", action="store_true",
+                    help="time the scalar-semantics forward (any block size, head_dim <= 256) instead of the MFMA "
+                         "kernel; adds its key-row traffic per launch and the rate it is read at")
     ap.add_argument("--packed-tiles", action="store_true",
                     help="pack the PARTIAL tiles once with the pre-pass kernel and time the forward on "
                          "packed tiles; also reports the pre-pass kernel against the HBM roofline")
@@ -411,6 +432,32 @@ def main(argv=None):
                        "frac": nbytes / (us * 1e-6) / 1e9 / 8000.0, "bytes_per_launch": nbytes,
                        "us_per_launch": us, "tiles": int(pm.shape[0]),
                        "note": "launch plus allocation of the output by the caller's allocator included"}
+        # the same kernel where it is bound by HBM and not by the launch: 65536 random tiles of this
+        # workload's shape, more than the 256 MB of last-level cache hold (kernel time from events,
+        # output preallocated through the raw entry point)
+        NBIG = 65536
+        big = torch.rand(NBIG, pm.shape[1], pm.shape[2], device=dev) < 0.5
+        words = torch.empty(NBIG, pm.shape[1], pm.shape[2] // 32, dtype=torch.int32, device=dev)
+        lib = omni_attn_capi.load_library()
+
+        def pack_big():
+            rc = lib.omni_attn_pack_partial_masks_gfx950(big.data_ptr(), words.data_ptr(), NBIG, pm.shape[1],
+                                                         pm.shape[2], stream.cuda_stream)
+            assert rc == 0, rc
+
+        for _ in range(5):
+            pack_big()
+        a.record(stream)
+        for _ in range(20):
+            pack_big()
+        b.record(stream)
+        torch.cuda.synchronize()
+        us_big = a.elapsed_time(b) * 1e3 / 20
+        nbytes_big = big.numel() + big.numel() // 8
+        pack_report["large"] = {"tiles": NBIG, "bytes_per_launch": nbytes_big, "us_per_launch": us_big,
+                                "achieved": nbytes_big / (us_big * 1e-6) / 1e9, "unit": "GB/s",
+                                "frac": nbytes_big / (us_big * 1e-6) / 1e9 / 8000.0}
+        del big, words
 
     bwd_state = None
     if args.backward:
@@ -429,6 +476,9 @@ def main(argv=None):
             omni_attn_capi.bwd(q, k, v, o, dout, lse, dq, dk, dv, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE,
                                S, pidx, None if bits is not None else pm, bits, workspace=ws,
                                stream=stream.cuda_stream)
+        elif args.generic_kernel:
+            omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, pidx, pm,
+                               stream=stream.cuda_stream, generic=True)
         elif bits is not None:
             omni_attn_capi.fwd(q, k, v, o, lse, nb, idx, tys, m.Q_BLOCK_SIZE, m.KV_BLOCK_SIZE, S, pidx, None,
                                stream=stream.cuda_stream, partial_bits=bits)
@@ -535,6 +585,16 @@ def main(argv=None):
     }
     if args.backward:
         out["config"]["pass"] = "backward (dQ kernel + dK/dV kernel), 10*QB*KB*D flop per listed block"
+    if args.generic_kernel:
+        # Every query row reads the K row (twice: maximum pass and weight pass) and the V row of every
+        # key it visits; nothing is shared between rows except through the caches.
+        pairs = visited_pairs(m)
+        nbytes = pairs * 3 * D * 2
+        out["config"]["kernel"] = "fwd_generic_kernel (one wave per query row, two passes, fp32)"
+        out["generic_kernel"] = {"bound": "l2", "row_key_pairs": pairs, "algorithmic_bytes": nbytes,
+                                 "achieved": nbytes / (avg_kernel_ms * 1e-3) / 1e9, "unit": "GB/s",
+                                 "note": "K (two passes) and V rows per visited (query row, key) pair; served by "
+                                         "L2 and L1, compulsory HBM bytes are 4*B*H*S*D*2"}
     if pack_report is not None:
         out["mask_pack"] = pack_report
         out["config"]["partial_tiles"] = "packed once by the pre-pass kernel"

@@ -85,7 +85,8 @@ enum omni_attn_status {
  *                    here an index outside [0, P) means "no bits stored".
  *   Tq               number of query blocks, must equal ceil(S_pad / QB).
  *   seqlen_orig      rows >= seqlen_orig are written as zeros (lse -inf); keys
- *                    >= seqlen_orig are never attended (attn_naive.cu:64-72, :113).
+ *                    >= seqlen_orig are never attended (attn_naive.cu:64-72, :113).  Those rows
+ *                    of q, k and v are never read: the padding may hold anything.
  *   softcap          0 = off (the reference's operator).  > 0: the scaled score x = q.k / sqrt(D)
  *                    is replaced by softcap * tanh(x / softcap) before the mask and the softmax,
  *                    the score_mod Transfusion's attention layer passes to flex_attention
@@ -178,7 +179,9 @@ int omni_attn_fwd_packed_gfx950(const void* q, const void* k, const void* v, voi
  *                     bytes (two floats per row), 4-byte aligned; holds -rowsum(dout . o) and
  *                     the rows' exponent offsets between the two kernels of the backward.
  *                     Contents before and after the call are meaningless.
- * Limits beyond the forward's: Tq * ceil(max_blocks / 64) <= 4096 (OMNI_ATTN_ERR_TOO_LARGE).
+ * Limits beyond the forward's: Tq * ceil(max_blocks / 64) <= 4096 (2602 at head_dim 128 with 128-key
+ * blocks), else OMNI_ATTN_ERR_TOO_LARGE.
+ * Rows at or beyond seqlen_orig of q, k, v, o and dout are never read (the padding may hold anything).
  * Two kernels are enqueued on `stream`; nothing is allocated; results are bitwise reproducible.
  */
 size_t omni_attn_bwd_workspace_bytes(int B, int H, int S_pad);
@@ -205,6 +208,10 @@ int omni_attn_bwd_gfx950(const void* q, const void* k, const void* v, const void
  * (4 194 304), else OMNI_ATTN_ERR_SCRATCH_LIMIT.  Calls no hipMalloc / hipFree or any other
  * allocating routine.  All calls on one GPU share that GPU's array: calls that overlap in time
  * on one GPU (different streams, different threads) race and must be serialised by the caller.
+ * Before recording a call into a HIP graph make one eager call with the same dtype, head_dim, block
+ * sizes and soft-cap setting on that device: the first call per device looks up the array's address
+ * and the device's topology, the first call per kernel instance raises that instance's dynamic-LDS
+ * limit -- none of them a stream operation.
  */
 size_t omni_attn_bwd_noalloc_max_rows(void);
 int omni_attn_bwd_noalloc_gfx950(const void* q, const void* k, const void* v, const void* o,

@@ -38,6 +38,7 @@ struct GenericParams {
   const uint8_t* partial_masks;
   int num_partial;
   int S, D, Tq, Tk, max_blocks, QB, KB, seqlen;
+  int k_rows_16b;  // every row of K starts on a 16-byte boundary (base aligned, D a multiple of 8)
   long long rows;  // B * H * S
   float scale, softcap;
 };
@@ -138,7 +139,21 @@ __global__ void __launch_bounds__(64 * kRowsPerWorkgroup) fwd_generic_kernel(con
     }
     const uint16_t* krow = p.k + slab + size_t(kv) * p.D;
     float s = 0.f;
-    for (int d = 0; d < p.D; ++d) s = __builtin_fmaf(sq[w][d], to_float<BF16>(krow[d]), s);
+    if (p.k_rows_16b) {  // rows of K start on 16-byte boundaries: eight elements per load
+      typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+      const u32x4_t* k8 = reinterpret_cast<const u32x4_t*>(krow);
+      for (int d8 = 0; d8 < p.D / 8; ++d8) {
+        const u32x4_t kk = k8[d8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t pair = kk[e];
+          s = __builtin_fmaf(sq[w][8 * d8 + 2 * e], to_float<BF16>(uint16_t(pair & 0xffffu)), s);
+          s = __builtin_fmaf(sq[w][8 * d8 + 2 * e + 1], to_float<BF16>(uint16_t(pair >> 16)), s);
+        }
+      }
+    } else {
+      for (int d = 0; d < p.D; ++d) s = __builtin_fmaf(sq[w][d], to_float<BF16>(krow[d]), s);
+    }
     s *= p.scale;  // :88
     if (p.softcap > 0.f) s = tanhf(s / p.softcap) * p.softcap;
     return s;
@@ -248,6 +263,7 @@ extern "C" int omni_attn_fwd_generic_gfx950(const void* q, const void* k, const 
   p.rows = rows;
   p.scale = float(1.0 / std::sqrt(double(D)));
   p.softcap = softcap;
+  p.k_rows_16b = (D % 8 == 0) && (reinterpret_cast<uintptr_t>(k) & 15) == 0;
   const unsigned grid = unsigned((rows + kRowsPerWorkgroup - 1) / kRowsPerWorkgroup);
   const void* kern = dtype == OMNI_ATTN_DTYPE_BF16 ? reinterpret_cast<const void*>(fwd_generic_kernel<true>)
                                                    : reinterpret_cast<const void*>(fwd_generic_kernel<false>);
