@@ -179,8 +179,9 @@ int omni_attn_fwd_packed_gfx950(const void* q, const void* k, const void* v, voi
  *                     bytes (two floats per row), 4-byte aligned; holds -rowsum(dout . o) and
  *                     the rows' exponent offsets between the two kernels of the backward.
  *                     Contents before and after the call are meaningless.
- * Limits beyond the forward's: Tq * ceil(max_blocks / 64) <= 4096 (2602 at head_dim 128 with 128-key
- * blocks), else OMNI_ATTN_ERR_TOO_LARGE.
+ * No limits beyond the forward's (Tq * ceil(max_blocks / 64) must fit an int).  Metadata of more
+ * than 4096 64-slot words per (batch, head) slab (2602 at head_dim 128 with 128-key blocks) is
+ * scanned in windows of that many words by every dK/dV workgroup.
  * Rows at or beyond seqlen_orig of q, k, v, o and dout are never read (the padding may hold anything).
  * Two kernels are enqueued on `stream`; nothing is allocated; results are bitwise reproducible.
  */

@@ -17,7 +17,8 @@
 //                    second kernel).
 //   bwd_dkdv_kernel  one workgroup per KV block; finds the (query block, slot) pairs that list
 //                    it by scanning the slab's metadata (a bitmap of the matches is built in
-//                    LDS first, then visited in ascending order).  Each 32 keys have two waves
+//                    LDS -- in windows, where the metadata has more words than LDS holds --
+//                    and visited in ascending order).  Each 32 keys have two waves
 //                    with different work (weights and dV / dP, dS and dK), so two waves share
 //                    a SIMD.
 // Both use the forward's building blocks with the operands exchanged: every product is a
@@ -587,20 +588,14 @@ struct BwdDkdvTraits {
   static constexpr size_t kFixedBytes = kTileBytes + kHandBytes + kRowBytes;
   // per 64-slot word of a slab's metadata: the bitmap of the slots that list this KV block (8
   // bytes) and mode / tile index of the first (4 bytes).  The launch asks for the words its
-  // metadata needs, so small problems fit two workgroups per compute unit.
+  // metadata needs, so small problems fit two workgroups per compute unit; metadata with more
+  // words than fit is worked through in windows of kMaxBitmapWords.
   static constexpr size_t kLdsLimit = size_t(160) * 1024;
   static constexpr int kMaxBitmapWords =
       (kLdsLimit - kFixedBytes) / 12 < 4096 ? int((kLdsLimit - kFixedBytes) / 12) : 4096;
   static constexpr size_t lds_bytes(size_t bitmap_words) { return kFixedBytes + bitmap_words * 12; }
   static constexpr size_t kLdsBytes = lds_bytes(kMaxBitmapWords);
 };
-
-// 64-slot words of match bitmap the dK/dV kernel of a (head_dim, KV block) pair can hold.
-constexpr int bwd_max_bitmap_words(int D, int KB) {
-  return D == 128 ? (KB == 128 ? BwdDkdvTraits<128, 128>::kMaxBitmapWords : BwdDkdvTraits<128, 64>::kMaxBitmapWords)
-       : D == 64  ? (KB == 128 ? BwdDkdvTraits<64, 128>::kMaxBitmapWords : BwdDkdvTraits<64, 64>::kMaxBitmapWords)
-                  : (KB == 128 ? BwdDkdvTraits<32, 128>::kMaxBitmapWords : BwdDkdvTraits<32, 64>::kMaxBitmapWords);
-}
 
 // Two 16-bit values of a word -> fp32 (exact).
 template <bool BF16>
@@ -657,7 +652,6 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
   float* const sNd = reinterpret_cast<float*>(lds_raw + Traits::kTileBytes + Traits::kHandBytes);  // [3 sets][STEP] -delta
   float* const sL2 = sNd + 3 * STEP;                                         // [3 sets][STEP] exponent offsets
   uint64_t* const sMatch = reinterpret_cast<uint64_t*>(sL2 + 3 * STEP);
-  int32_t* const sFirst = reinterpret_cast<int32_t*>(sMatch + p.Tq * ((p.max_blocks + 63) / 64));
 
   // Workgroup -> (slab, KV block): XCD x takes the slabs bh with bh % n_xcd == x one after the
   // other, so the workgroups that run together on an XCD read the Q and dO rows of one slab and
@@ -691,6 +685,9 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
   const size_t meta_slab = size_t(bh) * p.Tq;
   const int chunks = (p.max_blocks + 63) / 64;  // 64-slot words per query block
   const int n_words = p.Tq * chunks;
+  // words of the bitmap held in LDS at a time (what the launch sized the allocation for)
+  const int win_words = n_words < Traits::kMaxBitmapWords ? n_words : Traits::kMaxBitmapWords;
+  int32_t* const sFirst = reinterpret_cast<int32_t*>(sMatch + win_words);
 
   // This lane's key as B operand: K for a weight wave, V for a gradient wave (zeros for a key
   // beyond the sequence).
@@ -704,45 +701,53 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
     }
   }
 
-  // Pass 1: which (query block, slot) pairs list this KV block (after the forward's clamping of
+  // The scan: which (query block, slot) pairs list this KV block (after the forward's clamping of
   // the block index) with a type the forward would visit?  One 64-bit word per query block and 64
   // slots; a wave takes one word at a time.  Mode and tile index of a word's first match are
-  // kept beside it (a list names a block once, except for duplicates and clamped indices).
-  for (int word = w; word < n_words; word += NW) {
-    const int qb = word / chunks, ch = word - qb * chunks;
-    int nb = load_uniform(p.kv_num_blocks + meta_slab + qb);
-    nb = nb < 0 ? 0 : (nb > p.max_blocks ? p.max_blocks : nb);
-    const int slot = ch * 64 + lane;
-    bool hit = false;
-    int32_t info = 0;
-    if (slot < nb) {
-      const size_t o = (meta_slab + qb) * p.max_blocks + slot;
-      const int32_t raw = p.kv_indices[o];
-      const int32_t idx = raw < 0 ? 0 : (raw >= p.Tk ? p.Tk - 1 : raw);
-      const int32_t ty = p.types[o];
-      const int32_t pid = has_partial ? p.partial_idx[o] : -1;
-      const int32_t mode = bwd_slot_mode(ty, pid, has_partial, p.num_partial);
-      hit = idx == kvb && mode != kMasked;
-      info = (mode == kPartial ? pid << 2 : 0) | mode;
+  // kept beside it (a list names a block once, except for duplicates and clamped indices).  The
+  // words [base, end) of the slab go to entries 0 .. end - base of the window; every wave of the
+  // workgroup calls this at the same point (the barriers are the workgroup's).
+  auto scan_window = [&](int base, int end) {
+    __syncthreads();  // nobody reads the previous window any more
+    for (int word = base + w; word < end; word += NW) {
+      const int qb = word / chunks, ch = word - qb * chunks;
+      int nb = load_uniform(p.kv_num_blocks + meta_slab + qb);
+      nb = nb < 0 ? 0 : (nb > p.max_blocks ? p.max_blocks : nb);
+      const int slot = ch * 64 + lane;
+      bool hit = false;
+      int32_t info = 0;
+      if (slot < nb) {
+        const size_t o = (meta_slab + qb) * p.max_blocks + slot;
+        const int32_t raw = p.kv_indices[o];
+        const int32_t idx = raw < 0 ? 0 : (raw >= p.Tk ? p.Tk - 1 : raw);
+        const int32_t ty = p.types[o];
+        const int32_t pid = has_partial ? p.partial_idx[o] : -1;
+        const int32_t mode = bwd_slot_mode(ty, pid, has_partial, p.num_partial);
+        hit = idx == kvb && mode != kMasked;
+        info = (mode == kPartial ? pid << 2 : 0) | mode;
+      }
+      const uint64_t bits = __builtin_amdgcn_ballot_w64(hit);
+      if (lane == 0) sMatch[word - base] = bits;
+      if (bits != 0 && lane == __builtin_ctzll(bits)) sFirst[word - base] = info;
     }
-    const uint64_t bits = __builtin_amdgcn_ballot_w64(hit);
-    if (lane == 0) sMatch[word] = bits;
-    if (bits != 0 && lane == __builtin_ctzll(bits)) sFirst[word] = info;
-  }
-  __syncthreads();
+    __syncthreads();
+  };
 
   const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   f32x16_t acc[DT];  // dV^T of a weight wave, dK^T of a gradient wave
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16;
 
-  // Pass 2: the matches in ascending (query block, slot) order, each as NSTEPS steps of STEP
+  // The walk: the matches in ascending (query block, slot) order, each as NSTEPS steps of STEP
   // query rows, skipping steps beyond the sequence and CAUSAL steps entirely above the diagonal.
   // Inside a match the next step is the previous one moved on by STEP query rows (a CAUSAL step
   // that is valid stays valid further down; only the end of the sequence can end a match early):
   // that path is a handful of scalar instructions; the bitmap is only read at the first step of a
-  // match.
+  // match.  The generator ends at the end of the window LDS holds and goes on from there once the
+  // next window has been scanned.
   int gw = -1, g_qb = 0, g_ch = -1;  // word gw = (g_qb, g_ch)
+  int win_base = 0, win_end = win_words;  // the words of the slab the window holds
+  scan_window(0, win_end);
   uint64_t gbits = 0;
   bool g_first = true;
   BwdStepInfo g_last = {0, kMasked, -1, 0, 0, false};
@@ -758,12 +763,12 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
     g_last.valid = false;
     for (;;) {
       while (gbits == 0) {
-        if (++gw >= n_words) return g_last;
+        if (++gw >= win_end) return g_last;
         if (++g_ch == chunks) {
           g_ch = 0;
           ++g_qb;
         }
-        const uint64_t m = sMatch[gw];
+        const uint64_t m = sMatch[gw - win_base];
         // (readfirstlane returns a signed int: go through uint32_t so that bit 31 does not sign-extend)
         gbits = (uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(m >> 32))))) << 32) |
                 uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(m)))));
@@ -771,7 +776,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
       }
       int mode, pid;
       if (g_first) {
-        const int32_t info = __builtin_amdgcn_readfirstlane(sFirst[gw]);
+        const int32_t info = __builtin_amdgcn_readfirstlane(sFirst[gw - win_base]);
         mode = info & 3;
         pid = mode == kPartial ? info >> 2 : -1;
       } else {  // a further match in the same 64 slots
@@ -1009,54 +1014,63 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
 
   // Iteration j: the weight waves do step j, the gradient waves step j - 1.  The two roles
   // run separate copies of the loop (same trip count, one barrier per trip), so that each keeps
-  // its accumulators in place.
+  // its accumulators in place.  Metadata of more words than the bitmap holds takes several
+  // windows: the steps of a window are worked off completely before the next one is scanned.
   auto run = [&](auto role_c) {
     constexpr bool GRAD = decltype(role_c)::value;
     const BwdStepInfo none = {0, kMasked, -1, 0, 0, false};
-    BwdStepInfo prev = none, cur = next_step();
-    int s_prev = 2, s_cur = 0, s_nxt = 1;  // tile sets of steps j - 1, j, j + 1
-    if (cur.valid) {
-      if constexpr (!GRAD) load_q(cur, 0); else load_do(cur, 0);
-    }
-    for (int j = 0; cur.valid || prev.valid; ++j) {
-      const BwdStepInfo nxt = cur.valid ? next_step() : none;
-      // mask words of this lane's key: bit i of word u = query row row0 + 32 u + i attends it
-      uint32_t kw[NSUB];
-#pragma unroll
-      for (int u = 0; u < NSUB; ++u) kw[u] = 0;
-      if constexpr (!GRAD) {
-        if (cur.valid) {
-#pragma unroll
-          for (int u = 0; u < NSUB; ++u) {
-            uint32_t m = key_live ? 0xffffffffu : 0u;
-            if (cur.mode == kCausal) {  // rows at or after the key
-              const int n = key - (cur.row0 + 32 * u);
-              m &= n <= 0 ? 0xffffffffu : (n >= 32 ? 0u : (0xffffffffu << (n & 31)));
+    for (;;) {
+      BwdStepInfo prev = none, cur = next_step();
+      int s_prev = 2, s_cur = 0, s_nxt = 1;  // tile sets of steps j - 1, j, j + 1
+      if (cur.valid) {
+        if constexpr (!GRAD) load_q(cur, 0); else load_do(cur, 0);
+      }
+      for (int j = 0; cur.valid || prev.valid; ++j) {
+        const BwdStepInfo nxt = cur.valid ? next_step() : none;
+        // mask words of this lane's key: bit i of word u = query row row0 + 32 u + i attends it
+        uint32_t kw[NSUB];
+  #pragma unroll
+        for (int u = 0; u < NSUB; ++u) kw[u] = 0;
+        if constexpr (!GRAD) {
+          if (cur.valid) {
+  #pragma unroll
+            for (int u = 0; u < NSUB; ++u) {
+              uint32_t m = key_live ? 0xffffffffu : 0u;
+              if (cur.mode == kCausal) {  // rows at or after the key
+                const int n = key - (cur.row0 + 32 * u);
+                m &= n <= 0 ? 0xffffffffu : (n >= 32 ? 0u : (0xffffffffu << (n & 31)));
+              }
+              if (cur.mode == kPartial) m &= partial_column(cur.pid, cur.row0 + 32 * u - cur.blk * QB);
+              kw[u] = m >> (4 * g);
             }
-            if (cur.mode == kPartial) m &= partial_column(cur.pid, cur.row0 + 32 * u - cur.blk * QB);
-            kw[u] = m >> (4 * g);
           }
         }
-      }
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the tile this wave loaded has landed
-      __syncthreads();  // ... everybody's have; the hand-over of step j - 1 is written; the set
-                        // about to be overwritten (step j - 2) is no longer read
-      if constexpr (!GRAD) {
-        if (nxt.valid) load_q(nxt, s_nxt);
-        if (cur.valid) {
-          // (wave-uniform) a FULL step whose keys are all inside the sequence needs no mask
-          weight_step(s_cur, j & 1, kw, !(cur.mode == kFull && key_wave_min + 32 <= p.seqlen));
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the tile this wave loaded has landed
+        __syncthreads();  // ... everybody's have; the hand-over of step j - 1 is written; the set
+                          // about to be overwritten (step j - 2) is no longer read
+        if constexpr (!GRAD) {
+          if (nxt.valid) load_q(nxt, s_nxt);
+          if (cur.valid) {
+            // (wave-uniform) a FULL step whose keys are all inside the sequence needs no mask
+            weight_step(s_cur, j & 1, kw, !(cur.mode == kFull && key_wave_min + 32 <= p.seqlen));
+          }
+        } else {
+          if (nxt.valid) load_do(nxt, s_nxt);
+          if (prev.valid) grad_step(s_prev, (j + 1) & 1);
         }
-      } else {
-        if (nxt.valid) load_do(nxt, s_nxt);
-        if (prev.valid) grad_step(s_prev, (j + 1) & 1);
+        prev = cur;
+        cur = nxt;
+        const int t3 = s_prev;
+        s_prev = s_cur;
+        s_cur = s_nxt;
+        s_nxt = t3;
       }
-      prev = cur;
-      cur = nxt;
-      const int t3 = s_prev;
-      s_prev = s_cur;
-      s_cur = s_nxt;
-      s_nxt = t3;
+      if (__builtin_expect(win_end >= n_words, 1)) break;
+      // (rare) more words of metadata than the bitmap holds: the next window
+      win_base = win_end;
+      win_end = win_base + win_words < n_words ? win_base + win_words : n_words;
+      scan_window(win_base, win_end);
+      gw = win_base - 1;
     }
     __syncthreads();
     uint16_t* stage = lds16 + size_t(w) * 32 * D;
@@ -1098,7 +1112,8 @@ int launch_bwd_cap(const BwdParams& p, hipStream_t stream) {
   const unsigned slabs_per_xcd = unsigned(p.n_slabs + p.n_xcd - 1) / unsigned(p.n_xcd);
   BwdParams params = p;
   void* args[] = {&params};
-  const size_t dkdv_lds = TK::lds_bytes(size_t(p.Tq) * size_t((p.max_blocks + 63) / 64));
+  const size_t n_words = size_t(p.Tq) * size_t((p.max_blocks + 63) / 64);
+  const size_t dkdv_lds = TK::lds_bytes(n_words < size_t(TK::kMaxBitmapWords) ? n_words : size_t(TK::kMaxBitmapWords));
   const dim3 dkdv_grid(unsigned(p.n_xcd) * slabs_per_xcd * unsigned(p.Tk));
   const dim3 dq_grid(unsigned(p.n_xcd) * slabs_per_xcd * unsigned(p.Tq));
   e = hipLaunchKernel(reinterpret_cast<const void*>(kq), dq_grid, dim3(TQ::kThreads), args, TQ::kLdsBytes, stream);

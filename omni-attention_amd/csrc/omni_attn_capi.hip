@@ -236,9 +236,8 @@ int backward(const void* q, const void* k, const void* v, const void* o, const v
   if ((long long)S_pad * D > 0x7fffffffLL || total > 0x7fffffffLL / 2 || (long long)B * H * Tk > 0x7fffffffLL / 2 ||
       total * max_blocks > (1LL << 40) || (long long)num_partial * QB * KB > 0x7fffffffLL * 64)
     return OMNI_ATTN_ERR_TOO_LARGE;
-  // the dK/dV kernel keeps one bit per (query block, slot) of a slab in LDS
-  if ((long long)Tq * ((max_blocks + 63) / 64) > bwd_max_bitmap_words(D, KB))
-    return OMNI_ATTN_ERR_TOO_LARGE;
+  // the dK/dV kernel numbers the 64-slot words of a slab's metadata with an int
+  if ((long long)Tq * ((max_blocks + 63) / 64) > 0x7fffffffLL) return OMNI_ATTN_ERR_TOO_LARGE;
 
   BwdParams p;
   p.q = static_cast<const uint16_t*>(q);

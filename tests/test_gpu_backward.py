@@ -159,18 +159,14 @@ def test_slab_counts_that_do_not_divide_over_the_xcds(gpu_device):
         assert (got[3].float().cpu() - fwd_ref).abs().max().item() <= 1e-2
 
 
-def test_wide_block_lists_backward(gpu_device):
-    """Lists wider than 64 and 128 slots (most of them MASKED padding, the real blocks scattered over
-    the whole width): the metadata of a query block then spans several 64-slot words, in the dQ
-    kernel's register chunks and in the dK/dV kernel's match bitmap alike."""
-    gen = torch.Generator().manual_seed(105)
-    B, H, S, D, QB, KB, W = 1, 2, 512, 64, 128, 64, 150
+def scattered_lists(gen, H, S, QB, KB, W):
+    """Metadata of H heads whose lists are W slots wide, nearly all MASKED padding, with the real
+    blocks (FULL, CAUSAL and PARTIAL, about three quarters of the KV blocks) at random slots."""
     Tq, Tk = S // QB, S // KB
-    q, k, v, dout = (torch.randn(B, H, S, D, generator=gen).to(torch.float16) for _ in range(4))
-    nb = torch.zeros(B, H, Tq, dtype=torch.int32)
-    idx = torch.randint(0, Tk, (B, H, Tq, W), generator=gen, dtype=torch.int32)
-    tys = torch.zeros(B, H, Tq, W, dtype=torch.int32)  # MASKED
-    pidx = torch.full((B, H, Tq, W), -1, dtype=torch.int32)
+    nb = torch.zeros(1, H, Tq, dtype=torch.int32)
+    idx = torch.randint(0, Tk, (1, H, Tq, W), generator=gen, dtype=torch.int32)
+    tys = torch.zeros(1, H, Tq, W, dtype=torch.int32)  # MASKED
+    pidx = torch.full((1, H, Tq, W), -1, dtype=torch.int32)
     tiles = []
     for h in range(H):
         for qb in range(Tq):
@@ -188,13 +184,52 @@ def test_wide_block_lists_backward(gpu_device):
                 if ty == 3:
                     pidx[0, h, qb, s] = len(tiles)
                     tiles.append(torch.rand(QB, KB, generator=gen) < 0.5)
-    pm = torch.stack(tiles).to(torch.uint8)
+    return nb, idx, tys, pidx, torch.stack(tiles).to(torch.uint8)
+
+
+def test_wide_block_lists_backward(gpu_device):
+    """Lists wider than 64 and 128 slots (most of them MASKED padding, the real blocks scattered over
+    the whole width): the metadata of a query block then spans several 64-slot words, in the dQ
+    kernel's register chunks and in the dK/dV kernel's match bitmap alike."""
+    gen = torch.Generator().manual_seed(105)
+    B, H, S, D, QB, KB, W = 1, 2, 512, 64, 128, 64, 150
+    q, k, v, dout = (torch.randn(B, H, S, D, generator=gen).to(torch.float16) for _ in range(4))
+    nb, idx, tys, pidx, pm = scattered_lists(gen, H, S, QB, KB, W)
     got = run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, S, pidx, pm, device=gpu_device)
     dense = dense_mask_from_blocks(nb, idx, tys, QB, KB, S, S, pidx, pm, seqlen_orig=S)
     ref = attention_dense_grads(q, k, v, dense, dout)
     check_grads(got[:3], ref, torch.float16, "wide lists")
     fwd_ref, _ = attention_dense_fp32(q, k, v, dense)
     assert (got[3].float().cpu() - fwd_ref).abs().max().item() <= 2e-3
+
+
+@pytest.mark.parametrize("dtype,D,QB,KB,S,W,windows", [
+    (torch.bfloat16, 128, 128, 128, 2048, 64 * 400, 3),   # 16 x 400 = 6400 words, 2602 held at a time
+    (torch.float16, 64, 64, 64, 1024, 64 * 300, 2),       # 16 x 300 = 4800 words, 4096 at a time
+    (torch.float16, 128, 64, 64, 1024, 64 * 300, 2),
+])
+def test_metadata_beyond_one_bitmap_window(dtype, D, QB, KB, S, W, windows, gpu_device):
+    """More 64-slot words of metadata per slab than the dK/dV kernel's match bitmap holds in LDS:
+    the kernel scans and walks them window by window (the boundaries fall inside a query block's
+    list), and the gradients are those of the same blocks in a narrow list."""
+    gen = torch.Generator().manual_seed(115)
+    H = 2
+    words = (S // QB) * (W // 64)
+    assert windows == -(-words // (2602 if (D, KB) == (128, 128) else 4096))
+    q, k, v, dout = (torch.randn(1, H, S, D, generator=gen).to(dtype) for _ in range(4))
+    nb, idx, tys, pidx, pm = scattered_lists(gen, H, S, QB, KB, W)
+    got = run_fwd_bwd(q, k, v, dout, nb, idx, tys, QB, KB, S - 5, pidx, pm, device=gpu_device, softcap=0.0)
+    dense = dense_mask_from_blocks(nb, idx, tys, QB, KB, S, S, pidx, pm, seqlen_orig=S - 5)
+    check_grads(got[:3], attention_dense_grads(q, k, v, dense, dout), dtype, f"{words} words of metadata")
+    fwd_ref, _ = attention_dense_fp32(q, k, v, dense)
+    assert (got[3].float().cpu() - fwd_ref).abs().max().item() <= (1e-2 if dtype == torch.bfloat16 else 2e-3)
+    # the same blocks packed to the front of a list one window holds: bit-identical gradients
+    order = torch.argsort((tys == 0).to(torch.int8), dim=-1, stable=True)[..., :S // KB]
+    narrow = [torch.gather(t, -1, order).contiguous() for t in (idx, tys, pidx)]
+    nb2 = (tys != 0).sum(-1).to(torch.int32)
+    got2 = run_fwd_bwd(q, k, v, dout, nb2, narrow[0], narrow[1], QB, KB, S - 5, narrow[2], pm, device=gpu_device)
+    for name, a, b in zip(("dQ", "dK", "dV"), got[:3], got2[:3]):
+        assert torch.equal(a, b), f"{name} differs between the wide and the narrow list"
 
 
 def test_c2_full_size_backward_on_sampled_slabs(gpu_device):
