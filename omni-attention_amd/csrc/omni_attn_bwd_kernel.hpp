@@ -707,28 +707,39 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
   // kept beside it (a list names a block once, except for duplicates and clamped indices).  The
   // words [base, end) of the slab go to entries 0 .. end - base of the window; every wave of the
   // workgroup calls this at the same point (the barriers are the workgroup's).
-  auto scan_window = [&](int base, int end) {
+  auto scan_window = [&](auto scan_c, int base, int end) {
     __syncthreads();  // nobody reads the previous window any more
-    for (int word = base + w; word < end; word += NW) {
-      const int qb = word / chunks, ch = word - qb * chunks;
-      int nb = load_uniform(p.kv_num_blocks + meta_slab + qb);
-      nb = nb < 0 ? 0 : (nb > p.max_blocks ? p.max_blocks : nb);
-      const int slot = ch * 64 + lane;
-      bool hit = false;
-      int32_t info = 0;
-      if (slot < nb) {
-        const size_t o = (meta_slab + qb) * p.max_blocks + slot;
-        const int32_t raw = p.kv_indices[o];
-        const int32_t idx = raw < 0 ? 0 : (raw >= p.Tk ? p.Tk - 1 : raw);
-        const int32_t ty = p.types[o];
-        const int32_t pid = has_partial ? p.partial_idx[o] : -1;
-        const int32_t mode = bwd_slot_mode(ty, pid, has_partial, p.num_partial);
-        hit = idx == kvb && mode != kMasked;
-        info = (mode == kPartial ? pid << 2 : 0) | mode;
+    // A wave takes SCAN consecutive words per pass and has the loads of all of them in flight
+    // together (every slot inside the list's width is loaded; kv_num_blocks cuts afterwards).
+    // The first window, scanned while few registers are live, takes four; later ones one.
+    constexpr int SCAN = decltype(scan_c)::value;
+    for (int word0 = base + w * SCAN; word0 < end; word0 += NW * SCAN) {
+      int32_t raw[SCAN], ty[SCAN], pid[SCAN], nbv[SCAN];
+#pragma unroll
+      for (int u = 0; u < SCAN; ++u) {
+        const int word = word0 + u < end ? word0 + u : end - 1;  // (a repeat of the last word: ignored below)
+        const int qb = word / chunks, ch = word - qb * chunks;
+        const int slot = ch * 64 + lane;
+        const size_t o = (meta_slab + qb) * p.max_blocks + (slot < p.max_blocks ? slot : p.max_blocks - 1);
+        raw[u] = p.kv_indices[o];
+        ty[u] = p.types[o];
+        pid[u] = has_partial ? p.partial_idx[o] : -1;
+        nbv[u] = p.kv_num_blocks[meta_slab + qb];
       }
-      const uint64_t bits = __builtin_amdgcn_ballot_w64(hit);
-      if (lane == 0) sMatch[word - base] = bits;
-      if (bits != 0 && lane == __builtin_ctzll(bits)) sFirst[word - base] = info;
+#pragma unroll
+      for (int u = 0; u < SCAN; ++u) {
+        const int word = word0 + u;
+        if (word >= end) break;
+        const int ch = word % chunks;
+        const int nb = nbv[u] < 0 ? 0 : (nbv[u] > p.max_blocks ? p.max_blocks : nbv[u]);
+        const int32_t idx = raw[u] < 0 ? 0 : (raw[u] >= p.Tk ? p.Tk - 1 : raw[u]);
+        const int32_t mode = bwd_slot_mode(ty[u], pid[u], has_partial, p.num_partial);
+        const bool hit = ch * 64 + lane < nb && idx == kvb && mode != kMasked;
+        const int32_t info = (mode == kPartial ? pid[u] << 2 : 0) | mode;
+        const uint64_t bits = __builtin_amdgcn_ballot_w64(hit);
+        if (lane == 0) sMatch[word - base] = bits;
+        if (bits != 0 && lane == __builtin_ctzll(bits)) sFirst[word - base] = info;
+      }
     }
     __syncthreads();
   };
@@ -747,7 +758,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
   // next window has been scanned.
   int gw = -1, g_qb = 0, g_ch = -1;  // word gw = (g_qb, g_ch)
   int win_base = 0, win_end = win_words;  // the words of the slab the window holds
-  scan_window(0, win_end);
+  scan_window(IntC<4>{}, 0, win_end);
   uint64_t gbits = 0;
   bool g_first = true;
   BwdStepInfo g_last = {0, kMasked, -1, 0, 0, false};
@@ -1069,7 +1080,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
       // (rare) more words of metadata than the bitmap holds: the next window
       win_base = win_end;
       win_end = win_base + win_words < n_words ? win_base + win_words : n_words;
-      scan_window(win_base, win_end);
+      scan_window(IntC<1>{}, win_base, win_end);
       gw = win_base - 1;
     }
     __syncthreads();
