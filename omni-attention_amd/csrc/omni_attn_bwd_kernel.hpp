@@ -703,7 +703,7 @@ __global__ void __launch_bounds__(KB * 4, D == 128 ? 2 : 4) bwd_dkdv_kernel(cons
 
   // The scan: which (query block, slot) pairs list this KV block (after the forward's clamping of
   // the block index) with a type the forward would visit?  One 64-bit word per query block and 64
-  // slots; a wave takes one word at a time.  Mode and tile index of a word's first match are
+  // slots.  Mode and tile index of a word's first match are
   // kept beside it (a list names a block once, except for duplicates and clamped indices).  The
   // words [base, end) of the slab go to entries 0 .. end - base of the window; every wave of the
   // workgroup calls this at the same point (the barriers are the workgroup's).
