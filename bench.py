@@ -346,6 +346,86 @@ def operator_overhead(name, seed, dev, calls=200):
             "what": "omni_attention_shared_kv_swizzle(query, key, value, block_mask) vs omni_attn_fwd_gfx950"}
 
 
+# The reference's published grid (omni-attn-mma/logs/printed_mask.md:186-237): B=1, H=8, head_dim 64,
+# fp16, sequence / block size as below; the figures are its swizzle kernel's "TFLOPS" on an NVIDIA
+# GPU it does not name -- context, not a baseline for this metric.
+REFERENCE_GRID_PUBLISHED = {
+    "causal": {(512, 64): 4.57, (512, 128): 4.35, (1024, 64): 14.39, (1024, 128): 12.47,
+               (2048, 64): 31.69, (2048, 128): 32.27},
+    "interleaved": {(512, 64): 4.62, (512, 128): 3.38, (1024, 64): 13.19, (1024, 128): 12.24,
+                    (2048, 64): 28.17, (2048, 128): 33.60},
+}
+
+
+def reference_dense_flops(B: int, H: int, N: int, D: int) -> float:
+    """The flop count behind the reference's "TFLOPS": every one of the N x N score positions,
+    softmax and scaling included, whatever the mask leaves out
+    (omni-attn-mma/test_with_debug_data.py:35-54, compute_dense_attn_tflops)."""
+    qk = B * H * N * N * (2 * D - 1)
+    softmax = B * H * N * (N - 1) + 3 * B * H * N * N + B * H * N * (N - 1)
+    scaling = B * H * N * N
+    pv = B * H * N * D * (2 * N - 1)
+    return float(qk + softmax + scaling + pv)
+
+
+def reference_grid(dev, seed: int):
+    """The shapes of the reference's published table, timed the reference's way -- one wall-clock
+    sample around a call of the swizzle wrapper plus a synchronise, after one untimed call
+    (test_with_debug_data.py:152-162) -- and with HIP events around the kernel (median of 30)."""
+    import torch
+
+    import omni_attn_capi
+    import omni_attn_torch as oat
+
+    B, H, D = 1, 8, 64
+    rows = []
+    for kind in ("causal", "interleaved"):
+        for S in (512, 1024, 2048):
+            for blk in (64, 128):
+                gen = torch.Generator().manual_seed(seed)
+                q, k, v = (torch.randn(B, H, S, D, generator=gen).to(torch.float16).to(dev) for _ in range(3))
+                if kind == "causal":
+                    m = oat.create_causal_omni_block_mask(B, H, S, S, blk, blk, device=dev)
+                else:  # three segments: text, an image span that ends off the block grid, text
+                    pos = torch.tensor([[[0, S // 4, S // 4 + S // 8 + 5]]], dtype=torch.int64)
+                    m = oat.create_omni_block_mask_from_modality_positions(pos, B, H, S, S, blk, blk, device=dev)
+                oat.omni_attention_shared_kv_swizzle(q, k, v, m)
+                torch.cuda.synchronize()
+                t0 = time.time()
+                oat.omni_attention_shared_kv_swizzle(q, k, v, m)
+                torch.cuda.synchronize()
+                wall_ms = (time.time() - t0) * 1e3
+                o = torch.empty_like(q)
+                stream = torch.cuda.current_stream(dev)
+
+                def launch():
+                    omni_attn_capi.fwd(q, k, v, o, None, m.kv_num_blocks, m.kv_indices, m.block_mask_types, blk, blk,
+                                       S, m.partial_block_mask_indices, m.partial_block_masks,
+                                       stream=stream.cuda_stream)
+
+                for _ in range(20):
+                    launch()
+                ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(30)]
+                for a, b in ev:
+                    a.record(stream)
+                    launch()
+                    b.record(stream)
+                torch.cuda.synchronize()
+                kernel_ms = sorted(a.elapsed_time(b) for a, b in ev)[15]
+                dense = reference_dense_flops(B, H, S, D)
+                listed = int(m.kv_num_blocks.sum().item())
+                rows.append({"mask": kind, "seq_len": S, "block": blk, "listed_blocks": listed,
+                             "wall_ms_one_call": wall_ms, "kernel_ms_median": kernel_ms,
+                             "dense_equivalent_tflops_wall": dense / (wall_ms * 1e-3) / 1e12,
+                             "dense_equivalent_tflops_kernel": dense / (kernel_ms * 1e-3) / 1e12,
+                             "effective_tflops_kernel": 4.0 * blk * blk * D * listed / (kernel_ms * 1e-3) / 1e12,
+                             "reference_published_swizzle_tflops": REFERENCE_GRID_PUBLISHED[kind][(S, blk)]})
+    return {"grid": "the reference's published shapes: B=1 H=8 head_dim 64 fp16, seq_len / block as listed",
+            "note": "dense-equivalent TFLOPS by the reference's formula (all N x N positions, softmax included); "
+                    "the published figures are from an NVIDIA GPU the reference does not name",
+            "rows": rows}
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -376,6 +456,8 @@ def main(argv=None):
                          "command shows what FETCH_SIZE / WRITE_SIZE read for a known traffic")
     ap.add_argument("--sweep-bands", action="store_true",
                     help="instead of the workload: kernel time against the number of listed blocks")
+    ap.add_argument("--reference-grid", action="store_true",
+                    help="instead of the workload: the shapes of the reference's published table, timed its way")
     args = ap.parse_args(argv)
     if args.kernel_source_hash:
         print(kernel_source_hash())
@@ -398,6 +480,9 @@ def main(argv=None):
     omni_attn_capi.load_library()  # fail loudly when the HIP library is missing
     if args.sweep_bands:
         print(json.dumps(band_sweep(dev, min(args.steps, 30), min(args.warmup, 5))))
+        return 0
+    if args.reference_grid:
+        print(json.dumps(reference_grid(dev, args.seed)))
         return 0
 
     w = make_workload(args.workload, seed=args.seed)

@@ -69,3 +69,19 @@ def test_json_line_has_the_contract_fields(gpu_device):
     for name in ("c1_causal", "c2_interleaved"):
         op = d["operator"][name]
         assert op["operator_ms_per_call"] >= op["kernel_ms"] * 0.9 and op["capi_ms_per_call"] > 0
+
+
+def test_reference_flop_count_reproduces_the_reference_printed_figures():
+    """The dense-equivalent flop count of bench.py --reference-grid against figures the reference
+    printed with its own (omni_attention_report.pdf, appendix: seq 2048, B=1 H=8 D=64: swizzle
+    0.31 ms = 28.10 TFLOPS, shared_kv 0.48 ms = 18.39, simple 66.68 ms = 0.13; ms.md:19-24: seq 1024,
+    shared_kv 0.25 ms = 8.73).  The times are printed to two digits, hence the intervals."""
+    import bench
+    f2048 = bench.reference_dense_flops(1, 8, 2048, 64)
+    f1024 = bench.reference_dense_flops(1, 8, 1024, 64)
+    assert f2048 / 0.315e-3 / 1e12 <= 28.10 <= f2048 / 0.305e-3 / 1e12
+    assert f2048 / 0.485e-3 / 1e12 <= 18.39 <= f2048 / 0.475e-3 / 1e12
+    assert abs(f2048 / 66.68e-3 / 1e12 - 0.13) < 0.005
+    assert f1024 / 0.255e-3 / 1e12 <= 8.73 <= f1024 / 0.245e-3 / 1e12
+    assert set(bench.REFERENCE_GRID_PUBLISHED) == {"causal", "interleaved"}
+
