@@ -85,3 +85,16 @@ def test_reference_flop_count_reproduces_the_reference_printed_figures():
     assert f1024 / 0.255e-3 / 1e12 <= 8.73 <= f1024 / 0.245e-3 / 1e12
     assert set(bench.REFERENCE_GRID_PUBLISHED) == {"causal", "interleaved"}
 
+
+@pytest.mark.gpu
+def test_reference_grid_mode_covers_the_published_table(gpu_device):
+    r = subprocess.run([sys.executable, BENCH, "--reference-grid"], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    d = json.loads(r.stdout.strip().splitlines()[-1])
+    assert len(d["rows"]) == 12
+    assert {(x["mask"], x["seq_len"], x["block"]) for x in d["rows"]} == {
+        (m, s, b) for m in ("causal", "interleaved") for s in (512, 1024, 2048) for b in (64, 128)}
+    for x in d["rows"]:
+        assert x["listed_blocks"] > 0 and 0 < x["kernel_ms_median"] <= x["wall_ms_one_call"]
+        assert x["effective_tflops_kernel"] <= x["dense_equivalent_tflops_kernel"] * 1.01
+
